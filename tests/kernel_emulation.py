@@ -45,13 +45,15 @@ class EmulatedKernels:
             if 0 <= d < ids.shape[0] and 0 <= s < source.shape[0]:
                 ids[d] = source[s]
 
-    def rms_norm(self, x, weight, eps, offset, out, delta, rows):
+    def rms_norm(self, x, weight, eps, offset, out, delta, rows, delta_bias=None):
         self._count("rms_norm")
         if delta is not None and delta.dim() == 3:
             total = delta[0].to(torch.float32)
             for p in range(1, delta.shape[0]):
                 total = total + delta[p]
             delta = total
+        if delta_bias is not None:      # a row that comes with the pending contribution
+            delta = delta_bias.expand_as(x) if delta is None else delta.to(torch.float32) + delta_bias
         if rows is None:
             v = x.to(self.acc)
             if delta is not None:
@@ -132,11 +134,11 @@ class EmulatedKernels:
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
-                        plan=None):
+                        plan=None, softcap=0.0):
         self._count("paged_attention")
         n = qkv.shape[0]
         n_rep = num_heads // num_kv_heads
-        q_all = qkv.view(n, num_heads + 2 * num_kv_heads, head_dim)[:, :num_heads].to(self.acc)
+        q_all = qkv[:, :num_heads * head_dim].reshape(n, num_heads, head_dim).to(self.acc)
         pages = cache.shape[0]
         kview = cache[:, 0].view(pages, num_kv_heads, page_size, head_dim)
         vview = cache[:, 1].view(pages, num_kv_heads, head_dim, page_size)
@@ -157,6 +159,8 @@ class EmulatedKernels:
             if window:
                 allowed &= key[None, :] > pos[:, None] - window
             scores = torch.einsum("qhd,khd->hqk", q, k) * scale
+            if softcap:
+                scores = softcap * torch.tanh(scores / softcap)
             # keys outside the window may hold NaN of pages given back: mask by selection, not by addition
             scores = torch.where(allowed[None], scores, torch.full_like(scores, float("-inf")))
             probs = torch.softmax(scores, dim=-1)
@@ -166,6 +170,76 @@ class EmulatedKernels:
 
     def plan_paged_attention(self, *args):
         return None
+
+    def head_prepare(self, rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim, page_size,
+                     interleaved, norm_eps, values_are_keys, parts):
+        self._count("head_prepare")
+        n, width = rows.shape
+        if parts is not None:
+            total = parts[0]
+            for p in range(1, parts.shape[0]):
+                total = total + parts[p]
+            v = total.to(self.acc)
+        else:
+            v = rows.to(self.acc)
+        if bias is not None:
+            v = v + bias.to(self.acc)
+        v = v.clone()
+        r = num_heads + num_kv_heads
+        heads = v[:, :r * head_dim].reshape(n, r, head_dim).clone()
+        as_projected = heads[:, num_heads:].clone()
+        if inv_freq is not None:
+            half = inv_freq.shape[0]
+            ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]          # float32 angles
+            cos, sin = ang.cos().to(self.acc)[:, None, :], ang.sin().to(self.acc)[:, None, :]
+            if interleaved:
+                x1, x2 = heads[..., 0:2 * half:2].clone(), heads[..., 1:2 * half:2].clone()
+                heads[..., 0:2 * half:2] = x1 * cos - x2 * sin
+                heads[..., 1:2 * half:2] = x2 * cos + x1 * sin
+            else:
+                x1, x2 = heads[..., :half].clone(), heads[..., half:2 * half].clone()
+                heads[..., :half] = x1 * cos - x2 * sin
+                heads[..., half:2 * half] = x2 * cos + x1 * sin
+        if norm_eps is not None:
+            heads = heads * torch.rsqrt(heads.pow(2).mean(-1, keepdim=True) + norm_eps)
+        v[:, :r * head_dim] = heads.reshape(n, -1)
+        rows.copy_(v.to(rows.dtype))
+        if cache is not None:
+            page = (slots // page_size).long()
+            off = (slots % page_size).long()
+            k = rows[:, num_heads * head_dim:r * head_dim].reshape(n, num_kv_heads, head_dim)
+            if values_are_keys:
+                val = as_projected.to(rows.dtype)
+            else:
+                val = rows[:, r * head_dim:(r + num_kv_heads) * head_dim].reshape(n, num_kv_heads, head_dim)
+            kview = cache[:, 0].view(cache.shape[0], num_kv_heads, page_size, head_dim)
+            vview = cache[:, 1].view(cache.shape[0], num_kv_heads, head_dim, page_size)
+            kview[page, :, off, :] = k
+            vview[page, :, :, off] = val
+
+    def sigmoid_gate(self, a, gate, out):
+        self._count("sigmoid_gate")
+        out.copy_((a.to(self.acc) * torch.sigmoid(gate.to(self.acc))).to(out.dtype))
+
+    def copy_columns(self, src, out):
+        self._count("copy_columns")
+        out.copy_(src)
+
+    def stream_add(self, x, addend, delta, delta_bias):
+        self._count("stream_add")
+        v = x.to(self.acc)
+        if delta is not None:
+            if delta.dim() == 3:
+                total = delta[0]
+                for p in range(1, delta.shape[0]):
+                    total = total + delta[p]
+                delta = total
+            v = v + delta.to(self.acc)
+        if delta_bias is not None:
+            v = v + delta_bias.to(self.acc)
+        if addend is not None:
+            v = v + addend.to(self.acc)
+        x.copy_(v.to(x.dtype))
 
     def linear_splits(self, rows, out_features, in_features, dtype):
         return self.splits

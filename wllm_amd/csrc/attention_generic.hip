@@ -61,7 +61,8 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
                                const int* __restrict__ seg_ctx_len, T* __restrict__ out,
                                float* __restrict__ partial_o, float* __restrict__ partial_ml, int token_begin,
                                int max_chunks, int num_heads, int num_kv_heads, int head_dim, int page_size,
-                               int max_pages, float scale, int window, int group_begin) {
+                               int max_pages, float scale, int window, int group_begin, int q_stride,
+                               float softcap) {
     const int token = token_begin + blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
     const int seg = token_segment[token];
     const int q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
@@ -78,7 +79,7 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
     const int group = num_heads / num_kv_heads;
     const int g_count = min(kGroupMax, group - group_begin);   // heads of this pass
     const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
-    const int width = (num_heads + 2 * num_kv_heads) * head_dim;
+    const int width = q_stride;            // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * head_dim;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * head_dim;
     const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * head_dim;
@@ -150,7 +151,7 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
             float t = s[g];
             t += __shfl_xor(t, 1, kWave);
             t += __shfl_xor(t, 2, kWave);
-            const float sc = valid ? t * scale : -INFINITY;
+            const float sc = valid ? capped_score(t * scale, softcap) : -INFINITY;
             m[g] = wave_max(sc);
             const float p = valid ? expf(sc - m[g]) : 0.f;        // m is finite if any key of the tile is valid
             l[g] = wave_sum(c == 0 ? p : 0.f);
@@ -325,7 +326,8 @@ WLLM_API int wllm_paged_attention_generic(const void* qkv, const void* cache, in
                                           const int* seg_ctx_len, void* out, void* partial_o, void* partial_ml,
                                           int partial_tokens, int max_ctx_len, int n, int num_heads, int num_kv_heads,
                                           int head_dim, int page_size, int max_pages, float scale, int window,
-                                          hipStream_t stream) {
+                                          int q_stride, float softcap, hipStream_t stream) {
+    if (q_stride < num_heads * head_dim || softcap < 0.f) return -1;
     if (head_dim <= 0 || head_dim % 4 != 0 || head_dim > kMaxHeadDim || num_heads % num_kv_heads != 0) return -1;
     if (partial_tokens < 1 || max_ctx_len < 1 || !partial_o || !partial_ml) return -1;
     const int group = num_heads / num_kv_heads;
@@ -342,7 +344,7 @@ WLLM_API int wllm_paged_attention_generic(const void* qkv, const void* cache, in
     paged_attention_generic_kernel<T, NV, DPL, V4><<<grid, kWave * kWaves, smem, stream>>>(                              \
         static_cast<const T*>(qkv), static_cast<const T*>(cache), block_tables, token_segment, seg_q_start, seg_q_len,  \
         seg_ctx_len, static_cast<T*>(out), static_cast<float*>(partial_o), static_cast<float*>(partial_ml), t0,         \
-        max_chunks, num_heads, num_kv_heads, head_dim, page_size, max_pages, scale, window, gb)
+        max_chunks, num_heads, num_kv_heads, head_dim, page_size, max_pages, scale, window, gb, q_stride, softcap)
 #define LAUNCH_SIZES(T, V4)                         \
     if (nv == 4) LAUNCH(T, 4, 1, V4);               \
     else if (nv == 8) LAUNCH(T, 8, 2, V4);          \

@@ -63,7 +63,8 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                             const int* __restrict__ live_items, const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                             const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                             float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
-                            int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+                            int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
+                            int q_stride, float cap_scale, float softcap) {
     constexpr int DC = HD / 32;   // 32-wide chunks of the head for the score product
     constexpr int DT = HD / 16;   // 16-row tiles of out^T
     // Shared memory, a part for each wavefront, used four times: three workgroups share a compute
@@ -98,7 +99,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     // ---- This lane's queries are asked for first: they arrive while the addresses of the keys and
     //      values are worked out. ----
     const int group = num_heads / num_kv_heads;
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int width = q_stride;                     // elements between two tokens' query rows
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
     const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
@@ -218,7 +219,8 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             const int t2 = e / 4, v = e % 4;
             const int key = kbase + (V16 ? 8 * g + 4 * t2 + v : 16 * t2 + 4 * g + v);
             ok[e] = row_valid && key <= pos && key >= lo && key >= key_begin && key < key_end;
-            sv[e] = s[t2][v];
+            // with a cap the score is scaled and bent here, and `scale_log2e` is log2(e) alone
+            sv[e] = softcap > 0.f ? softcap * tanhf(s[t2][v] * cap_scale) : s[t2][v];
             if (ok[e]) tile_max = fmaxf(tile_max, sv[e]);
         }
         tile_max = max_across(max_across(tile_max, 16), 32);
@@ -460,6 +462,8 @@ struct AttentionArguments {
     int num_heads, num_kv_heads, page_size, max_pages;
     float scale_log2e;
     int window;
+    int q_stride;
+    float cap_scale, softcap;
     hipStream_t stream;
 };
 
@@ -467,7 +471,8 @@ template <int HD, bool V16>
 int launch_items(const AttentionArguments& a) {
     paged_attention_mfma_kernel<HD, V16><<<a.num_items, 256, 0, a.stream>>>(
         a.qkv, a.cache, a.block_tables, a.items, a.live_items, a.seg_q_start, a.seg_q_len, a.seg_ctx_len, a.out,
-        a.partial_o, a.partial_ml, a.num_heads, a.num_kv_heads, a.page_size, a.max_pages, a.scale_log2e, a.window);
+        a.partial_o, a.partial_ml, a.num_heads, a.num_kv_heads, a.page_size, a.max_pages, a.scale_log2e, a.window,
+        a.q_stride, a.cap_scale, a.softcap);
     return 0;
 }
 
@@ -498,14 +503,19 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
                                        int num_reduce_items, const int* seg_q_start, const int* seg_q_len,
                                        const int* seg_ctx_len, void* out, float* partial_o, float* partial_ml,
                                        int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
-                                       float scale, int window, hipStream_t stream) {
+                                       float scale, int window, int q_stride, float softcap, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         num_heads >= (1 << 16))       // an item holds a key/value head and a tile's first row in 16 bits each
         return -1;
+    if (q_stride < num_heads * head_dim || q_stride % 8 != 0 || softcap < 0.f) return -1;
+    // with a cap the kernel scales and bends the score itself; the softmax then works on final scores
+    const float in_exponent = softcap > 0.f ? 1.f : scale;
+    const float cap_scale = softcap > 0.f ? scale / softcap : 0.f;
     const AttentionArguments a = {static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items,
                                   live_items, num_items, reduce_items, num_reduce_items, seg_q_start, seg_q_len,
                                   seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads,
-                                  page_size, max_pages, scale * 1.4426950408889634f, window, stream};
+                                  page_size, max_pages, in_exponent * 1.4426950408889634f, window, q_stride, cap_scale,
+                                  softcap, stream};
     switch (head_dim) {
         case 32: return launch_all<32>(a);
         case 64: return launch_all<64>(a);

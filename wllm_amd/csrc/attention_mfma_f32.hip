@@ -38,7 +38,8 @@ paged_attention_f32_kernel(const float* __restrict__ qkv, const float* __restric
                            const int* __restrict__ block_tables, const int* __restrict__ items,
                            const int* __restrict__ live_items, float* __restrict__ out,
                            float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
-                           int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+                           int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
+                           int q_stride, float cap_scale, float softcap) {
     constexpr int DQ = HD / 4;                  // elements of a lane group's quarter of the head
     constexpr int DT = HD / 16;                 // 16-row tiles of out^T
     constexpr int kQStride = HD + 4;            // floats; rows 4 banks apart: 16 lanes' 16-byte reads meet no conflict
@@ -59,7 +60,7 @@ paged_attention_f32_kernel(const float* __restrict__ qkv, const float* __restric
     const int i = lane % 16, g = lane / 16;
 
     const int group = num_heads / num_kv_heads;
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int width = q_stride;         // elements between two tokens' query rows
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
     const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
@@ -144,7 +145,8 @@ paged_attention_f32_kernel(const float* __restrict__ qkv, const float* __restric
         for (int e = 0; e < 8; ++e) {
             const int key = kbase + 16 * (e / 4) + 4 * g + e % 4;
             ok[e] = row_valid && key <= pos && key >= lo && key >= key_begin && key < key_end;
-            pe[e] = s[e / 4][e % 4];
+            // with a cap the score is scaled and bent here, and `scale_log2e` is log2(e) alone
+            pe[e] = softcap > 0.f ? softcap * tanhf(s[e / 4][e % 4] * cap_scale) : s[e / 4][e % 4];
             if (ok[e]) tile_max = fmaxf(tile_max, pe[e]);
         }
         tile_max = max_across(max_across(tile_max, 16), 32);
@@ -316,7 +318,8 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
                                    const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                                    const int* __restrict__ seg_ctx_len, float* __restrict__ out,
                                    float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
-                                   int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+                                   int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
+                           int q_stride, float cap_scale, float softcap) {
     constexpr int DQ = HD / 4, DT = HD / 16;
     constexpr int SK = HD + 4, SV = kBlockKeys + 4;
     __shared__ __align__(16) float k_s[kBlockKeys * SK];
@@ -333,7 +336,7 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
     const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int width = q_stride;         // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
     const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
@@ -422,6 +425,10 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
 #pragma unroll
             for (int v = 0; v < 4; ++v) sv[4 * t2 + v] = sc[v];
         }
+        if (softcap > 0.f) {            // the score is scaled and bent here; `scale_log2e` is then log2(e) alone
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sv[e] = softcap * tanhf(sv[e] * cap_scale);
+        }
         const bool inside = kbase + kBlockKeys - 1 <= t_pos_min && kbase >= t_lo_max;
         if (!inside) {
 #pragma unroll
@@ -480,11 +487,13 @@ template <int HD>
 int launch_f32(const float* qkv, const float* cache, const int* block_tables, const int* items, const int* live_items,
                int num_items, const int* reduce_items, int num_reduce_items, const int* seg_q_start, const int* seg_q_len,
                float* out, float* partial_o, float* partial_ml, int num_heads, int num_kv_heads, int page_size,
-               int max_pages, float scale_log2e, int window, hipStream_t stream) {
+               int max_pages, float scale_log2e, int window, int q_stride, float cap_scale, float softcap,
+               hipStream_t stream) {
     if (num_items > 0)
         paged_attention_f32_kernel<HD><<<num_items, 256, 0, stream>>>(qkv, cache, block_tables, items, live_items, out,
                                                                       partial_o, partial_ml, num_heads, num_kv_heads,
-                                                                      page_size, max_pages, scale_log2e, window);
+                                                                      page_size, max_pages, scale_log2e, window,
+                                                                      q_stride, cap_scale, softcap);
     if (num_reduce_items > 0)
         attention_reduce_f32_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile / 4), HD, 0, stream>>>(
             reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, out, num_heads, num_kv_heads, scale_log2e);
@@ -500,15 +509,17 @@ WLLM_API int wllm_paged_attention_mfma_f32(const float* qkv, const float* cache,
                                            int num_reduce_items, const int* seg_q_start, const int* seg_q_len, float* out,
                                            float* partial_o, float* partial_ml, int num_heads, int num_kv_heads,
                                            int head_dim, int page_size, int max_pages, float scale, int window,
-                                           hipStream_t stream) {
+                                           int q_stride, float softcap, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         num_heads >= (1 << 16))       // an item holds a key/value head and a tile's first row in 16 bits each
         return -1;
-    const float scale_log2e = scale * 1.4426950408889634f;
+    if (q_stride < num_heads * head_dim || q_stride % 4 != 0 || softcap < 0.f) return -1;
+    const float scale_log2e = (softcap > 0.f ? 1.f : scale) * 1.4426950408889634f;
+    const float cap_scale = softcap > 0.f ? scale / softcap : 0.f;
 #define LAUNCH(HD)                                                                                                       \
     return launch_f32<HD>(qkv, cache, block_tables, items, live_items, num_items, reduce_items, num_reduce_items,         \
                           seg_q_start, seg_q_len, out, partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
-                          scale_log2e, window, stream)
+                          scale_log2e, window, q_stride, cap_scale, softcap, stream)
     switch (head_dim) {
         case 32: LAUNCH(32);
         case 64: LAUNCH(64);
@@ -530,17 +541,20 @@ WLLM_API int wllm_paged_attention_prefill_f32(const float* qkv, const float* cac
                                               int num_items, int rows_per_item, const int* seg_q_start, const int* seg_q_len,
                                               const int* seg_ctx_len, float* out, float* partial_o, float* partial_ml,
                                               int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
-                                              float scale, int window, hipStream_t stream) {
+                                              float scale, int window, int q_stride, float softcap, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         rows_per_item != 64)
         return -1;
+    if (q_stride < num_heads * head_dim || q_stride % 4 != 0 || softcap < 0.f) return -1;
     if (num_items <= 0) return 0;
-    const float scale_log2e = scale * 1.4426950408889634f;
+    const float scale_log2e = (softcap > 0.f ? 1.f : scale) * 1.4426950408889634f;
+    const float cap_scale = softcap > 0.f ? scale / softcap : 0.f;
 #define LAUNCH(HD)                                                                                                    \
     paged_attention_prefill_f32_kernel<HD><<<num_items, 256, 0, stream>>>(qkv, cache, block_tables, items, seg_q_start, \
                                                                           seg_q_len, seg_ctx_len, out, partial_o,        \
                                                                           partial_ml, num_heads, num_kv_heads, page_size, \
-                                                                          max_pages, scale_log2e, window);               \
+                                                                          max_pages, scale_log2e, window, q_stride,      \
+                                                                          cap_scale, softcap);                            \
     break
     switch (head_dim) {
         case 32: LAUNCH(32);

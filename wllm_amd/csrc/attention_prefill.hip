@@ -50,7 +50,8 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
                                const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                                const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                                float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
-                               int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+                               int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
+                               int q_stride, float cap_scale, float softcap) {
     constexpr int DC = HD / 32, DT = HD / 16;
     constexpr int SK = PrefillSmem<HD>::kStrideK, SV = PrefillSmem<HD>::kStrideV;
     __shared__ __align__(16) uint16_t k_s[kBlockKeys * SK];
@@ -68,7 +69,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
     const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int width = q_stride;         // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
     const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
@@ -245,6 +246,10 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             float sv[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) sv[e] = s[rt][e / 4][e % 4];
+            if (softcap > 0.f) {        // the score is scaled and bent here; `scale_log2e` is then log2(e) alone
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sv[e] = softcap * tanhf(sv[e] * cap_scale);
+            }
             // blocks that lie wholly inside every row's range need no mask (a wavefront-wide decision)
             const bool inside = kbase + kBlockKeys - 1 <= t_pos_min[rt] && kbase >= t_lo_max[rt];
             if (!inside) {
@@ -373,7 +378,8 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
                                    const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                                    const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                                    float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
-                                   int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+                                   int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
+                               int q_stride, float cap_scale, float softcap) {
     constexpr int DC = HD / 32, DT = HD / 16, CPR = HD / 8;       // CPR: 16-byte chunks of a key row
     constexpr int kKeyInstr = kBlockKeys * CPR / 64, kValInstr = HD * 4 / 64;    // wavefront loads per tile
     __shared__ __align__(16) uint16_t k_s0[kBlockKeys * HD], k_s1[kBlockKeys * HD];
@@ -391,7 +397,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
     const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int width = q_stride;         // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
     const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
@@ -555,6 +561,10 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
 #pragma unroll
             for (int v = 0; v < 4; ++v) sv[4 * t2 + v] = sc[v];
         }
+        if (softcap > 0.f) {            // the score is scaled and bent here; `scale_log2e` is then log2(e) alone
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sv[e] = softcap * tanhf(sv[e] * cap_scale);
+        }
 #pragma unroll
         for (int t = 0; t < DT; ++t) vf[t].u = *reinterpret_cast<const uint4*>(&v_s[v_lane + 16 * t * 4 * 8]);
         __builtin_amdgcn_sched_barrier(0);
@@ -627,18 +637,20 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
                                           const int* seg_q_len, const int* seg_ctx_len, void* out, float* partial_o,
                                           float* partial_ml, int num_heads,
                                           int num_kv_heads, int head_dim, int page_size, int max_pages, float scale,
-                                          int window, hipStream_t stream) {
+                                          int window, int q_stride, float softcap, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
         return -1;
     if (rows_per_item != 64) return -1;
+    if (q_stride < num_heads * head_dim || q_stride % 8 != 0 || softcap < 0.f) return -1;
     if (num_items <= 0) return 0;
-    const float scale_log2e = scale * 1.4426950408889634f;
+    const float scale_log2e = (softcap > 0.f ? 1.f : scale) * 1.4426950408889634f;
+    const float cap_scale = softcap > 0.f ? scale / softcap : 0.f;
     if (page_size >= 8 && (page_size & (page_size - 1)) == 0 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
 #define LAUNCH_DMA(HD)                                                                                              \
     paged_attention_prefill_dma_kernel<HD><<<num_items, kPrefillThreads, 0, stream>>>(                              \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
-        scale_log2e, window)
+        scale_log2e, window, q_stride, cap_scale, softcap)
         if (head_dim == 64) LAUNCH_DMA(64);
         else if (head_dim == 128) LAUNCH_DMA(128);
         else LAUNCH_DMA(256);
@@ -649,7 +661,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     paged_attention_prefill_kernel<HD, RTW><<<num_items, kPrefillThreads, 0, stream>>>(                             \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
-        scale_log2e, window)
+        scale_log2e, window, q_stride, cap_scale, softcap)
 #define LAUNCH(HD) LAUNCH_RTW(HD, 1)
     switch (head_dim) {
         case 32: LAUNCH(32); break;

@@ -119,6 +119,13 @@ __device__ __forceinline__ float stack_sum(const float* __restrict__ p, int spli
 // rescaling, which a probability does not need.
 __device__ __forceinline__ float exp2_probability(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// A score bent under a cap: cap * tanh(score / cap), which is the score itself near zero and never
+// beyond the cap; cap 0 leaves the score as it is.  Every attention kernel goes through this, on
+// the scaled score, before the maximum is taken.
+__device__ __forceinline__ float capped_score(float score, float cap) {
+    return cap > 0.f ? cap * tanhf(score / cap) : score;
+}
+
 // The activations of a gated feed-forward, by the number the host passes (the table `ACTIVATIONS` of
 // the Python side holds the same numbers): every kernel that applies one goes through `activate`,
 // so a new activation is one line here, one there, and a case in `WLLM_BY_ACTIVATION`.

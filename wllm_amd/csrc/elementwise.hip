@@ -60,8 +60,8 @@ constexpr int kNormPerThread = 8;    // elements a thread may keep in registers 
 
 template <typename TD, typename TO>
 __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits, size_t split_stride,
-                                const float* __restrict__ weight, const int* __restrict__ rows, TO* __restrict__ out,
-                                int hidden, float eps, float offset) {
+                                const float* __restrict__ dbias, const float* __restrict__ weight,
+                                const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps, float offset) {
     __shared__ float scratch[16];
     const int orow = blockIdx.x;
     const int irow = rows ? rows[orow] : orow;
@@ -78,10 +78,9 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
             float v = 0.f;
             if (i < hidden) {
                 v = xr[i];
-                if (dr) {
-                    v += delta_value(dr + i, splits, split_stride);
-                    if (!rows) xr[i] = v;
-                }
+                if (dr) v += delta_value(dr + i, splits, split_stride);
+                if (dbias) v += dbias[i];
+                if ((dr || dbias) && !rows) xr[i] = v;
             }
             keep[e] = v;
             ss += v * v;
@@ -89,10 +88,9 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
     } else {
         for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
             float v = xr[i];
-            if (dr) {
-                v += delta_value(dr + i, splits, split_stride);
-                if (!rows) xr[i] = v;
-            }
+            if (dr) v += delta_value(dr + i, splits, split_stride);
+            if (dbias) v += dbias[i];
+            if ((dr || dbias) && !rows) xr[i] = v;
             ss += v * v;
         }
     }
@@ -108,6 +106,7 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
         for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
             float v = xr[i];
             if (dr && rows) v += delta_value(dr + i, splits, split_stride);
+            if (dbias && rows) v += dbias[i];
             o[i] = from_float<TO>(v * inv * (offset + weight[i]));
         }
     }
@@ -121,9 +120,9 @@ template <typename T> struct alignas(4 * sizeof(T)) Quad { T v[4]; };
 
 template <typename TD, typename TO>
 __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits,
-                                    size_t split_stride, const float* __restrict__ weight,
-                                    const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps,
-                                    float offset) {
+                                    size_t split_stride, const float* __restrict__ dbias,
+                                    const float* __restrict__ weight, const int* __restrict__ rows,
+                                    TO* __restrict__ out, int hidden, float eps, float offset) {
     __shared__ float scratch[16];
     const int orow = blockIdx.x;
     const int irow = rows ? rows[orow] : orow;
@@ -163,8 +162,13 @@ __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict_
                 }
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v.v[k] += d.v[k];
-                if (!rows) *reinterpret_cast<Quad<float>*>(xr + i) = v;
             }
+            if (dbias) {        // a row that the pending contribution brings with it (a projection's bias)
+                const Quad<float> b = *reinterpret_cast<const Quad<float>*>(dbias + i);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v.v[k] += b.v[k];
+            }
+            if ((dr || dbias) && !rows) *reinterpret_cast<Quad<float>*>(xr + i) = v;
         }
         keep[e] = v;
 #pragma unroll
@@ -185,14 +189,14 @@ __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict_
 }
 
 WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, int splits, long long split_stride,
-                           const float* weight, const int* rows, void* out, int out_bf16, int num_out_rows,
+                           const float* dbias, const float* weight, const int* rows, void* out, int out_bf16, int num_out_rows,
                            int hidden, float eps, float offset, hipStream_t stream) {
     if (hidden % 4 == 0 && hidden <= 1024 * 4 * kNormGroups && (splits <= 1 || split_stride % 4 == 0)) {
         const int quads = hidden / 4;
         const int vthreads = quads >= 1024 ? 1024 : ((quads + 63) / 64) * 64;
 #define LAUNCH(TD, TO)                                                                                          \
     rms_norm_vec_kernel<TD, TO><<<num_out_rows, vthreads, 0, stream>>>(                                         \
-        x, static_cast<const TD*>(delta), splits, static_cast<size_t>(split_stride), weight, rows,             \
+        x, static_cast<const TD*>(delta), splits, static_cast<size_t>(split_stride), dbias, weight, rows,      \
         static_cast<TO*>(out), hidden, eps, offset)
         if (delta_bf16 && out_bf16) LAUNCH(bf16, bf16);
         else if (delta_bf16) LAUNCH(bf16, float);
@@ -204,8 +208,8 @@ WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, int spli
     const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 128 : 64));
 #define LAUNCH(TD, TO)                                                                                          \
     rms_norm_kernel<TD, TO><<<num_out_rows, threads, 0, stream>>>(x, static_cast<const TD*>(delta), splits,      \
-                                                                  static_cast<size_t>(split_stride), weight, rows, \
-                                                                  static_cast<TO*>(out), hidden, eps, offset)
+                                                                  static_cast<size_t>(split_stride), dbias, weight, \
+                                                                  rows, static_cast<TO*>(out), hidden, eps, offset)
     if (delta_bf16 && out_bf16) LAUNCH(bf16, bf16);
     else if (delta_bf16) LAUNCH(bf16, float);
     else if (out_bf16) LAUNCH(float, bf16);
@@ -427,14 +431,14 @@ WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* parts, i
 
 template <typename T, int ACT>
 __global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long long total,
-                                        int inter) {
+                                        int inter, long long out_stride) {
     const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
     for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
         const long long r = i / inter;
         const int c = static_cast<int>(i % inter);
         const float g = to_float(gate_up[r * 2 * inter + c]);
         const float u = to_float(gate_up[r * 2 * inter + inter + c]);
-        out[i] = from_float<T>(activate<ACT>(g) * u);
+        out[r * out_stride + c] = from_float<T>(activate<ACT>(g) * u);
     }
 }
 
@@ -443,11 +447,12 @@ __global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __rest
 // read once
 template <int ACT>
 __global__ void __launch_bounds__(256)
-gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, int rows, int inter) {
+gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, int rows, int inter,
+                               long long out_stride) {
     const int vecs = inter / 8;
     for (int r = blockIdx.y; r < rows; r += gridDim.y) {
         const bf16* src = gate_up + static_cast<size_t>(r) * 2 * inter;
-        bf16* dst = out + static_cast<size_t>(r) * inter;
+        bf16* dst = out + static_cast<size_t>(r) * out_stride;
         for (int v = blockIdx.x * 256 + threadIdx.x; v < vecs; v += gridDim.x * 256) {
             const uint4 g4 = load_streamed(src + v * 8);
             const uint4 u4 = load_streamed(src + inter + v * 8);
@@ -464,22 +469,25 @@ gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restric
     }
 }
 
+// `out_stride`: elements between two rows of out (inter, or more where out is a band of columns of a
+// wider buffer).
 WLLM_API int wllm_gated_activation(const void* gate_up, void* out, int is_bf16, int activation, int n, int inter,
-                                   hipStream_t stream) {
-    if (activation < 0 || activation >= kActivations) return -1;
+                                   long long out_stride, hipStream_t stream) {
+    if (activation < 0 || activation >= kActivations || out_stride < inter) return -1;
     const long long total = static_cast<long long>(n) * inter;
-    if (is_bf16 && inter % 8 == 0) {
+    if (is_bf16 && inter % 8 == 0 && out_stride % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
         const int vecs = inter / 8;
         const dim3 grid(vecs < 2048 ? (vecs + 255) / 256 : 8, n < 16384 ? n : 16384);
         WLLM_BY_ACTIVATION(activation, (gated_activation_bf16x8_kernel<ACT><<<grid, 256, 0, stream>>>(
-                                           static_cast<const bf16*>(gate_up), static_cast<bf16*>(out), n, inter)));
+                                           static_cast<const bf16*>(gate_up), static_cast<bf16*>(out), n, inter,
+                                           out_stride)));
         return launch_status();
     }
     long long blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
 #define LAUNCH(T)                                                                                                   \
     WLLM_BY_ACTIVATION(activation, (gated_activation_kernel<T, ACT><<<static_cast<int>(blocks), 256, 0, stream>>>( \
-                                       static_cast<const T*>(gate_up), static_cast<T*>(out), total, inter)))
+                                       static_cast<const T*>(gate_up), static_cast<T*>(out), total, inter, out_stride)))
     if (is_bf16) { LAUNCH(bf16); } else { LAUNCH(float); }
 #undef LAUNCH
     return launch_status();

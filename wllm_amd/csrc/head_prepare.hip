@@ -1,0 +1,247 @@
+// What lies between the projection of an attention block and its attention, for blocks that do
+// more there than rotate: per head a rotation (either pairing, the whole head or its first
+// elements), a unit norm of queries and keys, values that are the keys as projected, and columns
+// beyond the heads that only take their bias and the sum of their partial sums.  And three small
+// steps of the residual stream and of a block's output: a gate on the attention's result, a copy
+// into a band of columns, and a sum into the stream.  Everything here computes in float32.
+#include "common.h"
+
+constexpr int kPrepareWaves = 4;
+constexpr int kPrepareMaxHead = 256;
+constexpr int kPerLane = kPrepareMaxHead / kWave;
+
+// One workgroup per token, one wavefront per head at a time.  A row is
+//   [num_heads query heads | num_kv_heads key heads | num_kv_heads value heads, unless the values are the keys | extra]
+// of head_dim elements a head.  In the order of the steps, for every query and key head:
+//   1. the element is the row's (or the sum of the stack of partial sums `parts`), plus its bias;
+//   2. where the values are the keys, the key head as it is now goes to the cache's values;
+//   3. the first rotary_dim elements turn by position * inv_freq[j]: pair j is (2j, 2j + 1)
+//      (interleaved) or (j, j + rotary_dim / 2);
+//   4. with norm_eps >= 0 the head is divided by sqrt(mean of its squares + norm_eps);
+//   5. it is written back to the row, and a key head to the cache's keys.
+// Value heads of their own and the extra columns take step 1 only.  Keys lie in the cache as
+// [page_size, head_dim], values transposed as [head_dim, page_size].
+template <typename T>
+__global__ void __launch_bounds__(kWave * kPrepareWaves)
+head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict__ parts, int splits, size_t split_stride,
+                    const float* __restrict__ bias, const int* __restrict__ positions,
+                    const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ cache,
+                    long long num_pages, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
+                    int interleaved, float norm_eps, int values_are_keys, int page_size) {
+    __shared__ float staged[kPrepareWaves][kPrepareMaxHead];
+    const int token = blockIdx.x;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    T* row = rows + static_cast<size_t>(token) * row_width;
+    const float* prow = parts ? parts + static_cast<size_t>(token) * row_width : nullptr;
+    auto value = [&](int idx) -> float {
+        const float v = prow ? stack_sum(prow + idx, splits, split_stride) : to_float(row[idx]);
+        return bias ? v + bias[idx] : v;
+    };
+    const bool rewrite = bias || prow;
+    const float pos = static_cast<float>(positions[token]);
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * head_dim;
+    T* kpage = nullptr;
+    T* vpage = nullptr;
+    int off = 0;
+    if (cache) {
+        const int slot = slots[token];
+        const long long page = slot / page_size;
+        off = slot % page_size;
+        if (slot >= 0 && page < num_pages) {
+            kpage = cache + page * page_elems;
+            vpage = kpage + static_cast<size_t>(num_kv_heads) * page_size * head_dim;
+        }
+    }
+    // the lane's elements of a head are lane, lane + 64, ...; their angles do not depend on the head
+    const int half = rotary_dim / 2;
+    float sn[kPerLane], cs[kPerLane];
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+        const int e = lane + k * kWave;
+        sn[k] = 0.f;
+        cs[k] = 1.f;
+        if (inv_freq && e < rotary_dim) {
+            const int j = interleaved ? e >> 1 : (e < half ? e : e - half);
+            sincosf(pos * inv_freq[j], &sn[k], &cs[k]);
+        }
+    }
+    float* mine = staged[wave];
+    const int turned_heads = num_heads + num_kv_heads;
+    for (int head = wave; head < turned_heads; head += kPrepareWaves) {
+        const int base = head * head_dim;
+        const int kvh = head - num_heads;                 // >= 0: a key head
+        float v[kPerLane];
+#pragma unroll
+        for (int k = 0; k < kPerLane; ++k) {
+            const int e = lane + k * kWave;
+            v[k] = e < head_dim ? value(base + e) : 0.f;
+            if (e < head_dim) mine[e] = v[k];
+            if (values_are_keys && kvh >= 0 && vpage && e < head_dim)
+                vpage[(static_cast<size_t>(kvh) * head_dim + e) * page_size + off] = from_float<T>(v[k]);
+        }
+        // lanes read below what other lanes of the wavefront wrote above
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < kPerLane; ++k) {
+            const int e = lane + k * kWave;
+            if (inv_freq && e < rotary_dim) {
+                const bool first = interleaved ? (e & 1) == 0 : e < half;
+                const int partner = interleaved ? (e ^ 1) : (first ? e + half : e - half);
+                const float other = mine[partner];
+                float ra, rb;
+                rotate_pair(first ? v[k] : other, first ? other : v[k], sn[k], cs[k], ra, rb);
+                v[k] = first ? ra : rb;
+            }
+            ss += v[k] * v[k];
+        }
+        float inv = 1.f;
+        if (norm_eps >= 0.f) inv = rsqrtf(wave_sum(ss) / static_cast<float>(head_dim) + norm_eps);
+#pragma unroll
+        for (int k = 0; k < kPerLane; ++k) {
+            const int e = lane + k * kWave;
+            if (e < head_dim) {
+                const T r = from_float<T>(v[k] * inv);
+                row[base + e] = r;
+                if (kvh >= 0 && kpage) kpage[(static_cast<size_t>(kvh) * page_size + off) * head_dim + e] = r;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("" ::: "memory");
+    }
+    // value heads of their own
+    int done = turned_heads * head_dim;
+    if (!values_are_keys) {
+        if (rewrite || vpage) {
+            for (int idx = threadIdx.x; idx < num_kv_heads * head_dim; idx += blockDim.x) {
+                const int head = idx / head_dim, j = idx % head_dim;
+                T v = row[done + idx];
+                if (rewrite) {
+                    v = from_float<T>(value(done + idx));
+                    row[done + idx] = v;
+                }
+                if (vpage) vpage[(static_cast<size_t>(head) * head_dim + j) * page_size + off] = v;
+            }
+        }
+        done += num_kv_heads * head_dim;
+    }
+    // what lies beyond the heads
+    if (rewrite)
+        for (int idx = done + threadIdx.x; idx < row_width; idx += blockDim.x) row[idx] = from_float<T>(value(idx));
+}
+
+// Returns 0, a HIP error code, or -1 for sizes the kernel does not take.
+WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const float* parts, int splits,
+                               long long split_stride, const float* bias, const int* positions, const float* inv_freq,
+                               const int* slots, void* cache, long long num_pages, int n, int num_heads,
+                               int num_kv_heads, int head_dim, int rotary_dim, int interleaved, float norm_eps,
+                               int values_are_keys, int page_size, hipStream_t stream) {
+    const int heads = num_heads + (values_are_keys ? 1 : 2) * num_kv_heads;
+    if (head_dim <= 0 || head_dim > kPrepareMaxHead || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 != 0 ||
+        row_width < heads * head_dim || num_heads < 0 || num_kv_heads < 0 || page_size <= 0)
+        return -1;
+    if (inv_freq == nullptr && rotary_dim != 0) return -1;
+    if (n <= 0) return 0;
+#define LAUNCH(T)                                                                                                   \
+    head_prepare_kernel<T><<<n, kWave * kPrepareWaves, 0, stream>>>(                                                \
+        static_cast<T*>(rows), row_width, parts, splits, static_cast<size_t>(split_stride), bias, positions, inv_freq, \
+        slots, static_cast<T*>(cache), num_pages, num_heads, num_kv_heads, head_dim, rotary_dim, interleaved, norm_eps, \
+        values_are_keys, page_size)
+    if (is_bf16) LAUNCH(bf16);
+    else LAUNCH(float);
+#undef LAUNCH
+    return launch_status();
+}
+
+// ---- out[r, c] = a[r, c] * sigmoid(gate[r, c]); every operand has a row stride of its own, so the
+// gate may be a band of a wider row and the result a band of a wider buffer ----------------------
+template <typename T>
+__global__ void sigmoid_gate_kernel(const T* __restrict__ a, long long a_stride, const T* __restrict__ gate,
+                                    long long gate_stride, T* __restrict__ out, long long out_stride, int rows,
+                                    int cols) {
+    for (int r = blockIdx.y; r < rows; r += gridDim.y) {
+        const T* ar = a + r * a_stride;
+        const T* gr = gate + r * gate_stride;
+        T* o = out + r * out_stride;
+        for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x) {
+            const float g = to_float(gr[c]);
+            o[c] = from_float<T>(to_float(ar[c]) / (1.f + expf(-g)));
+        }
+    }
+}
+
+WLLM_API int wllm_sigmoid_gate(const void* a, long long a_stride, const void* gate, long long gate_stride, void* out,
+                               long long out_stride, int is_bf16, int rows, int cols, hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return 0;
+    const dim3 grid(cols < 4096 ? (cols + 255) / 256 : 16, rows < 16384 ? rows : 16384);
+    if (is_bf16)
+        sigmoid_gate_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(a), a_stride, static_cast<const bf16*>(gate),
+                                                            gate_stride, static_cast<bf16*>(out), out_stride, rows, cols);
+    else
+        sigmoid_gate_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(a), a_stride,
+                                                             static_cast<const float*>(gate), gate_stride,
+                                                             static_cast<float*>(out), out_stride, rows, cols);
+    return launch_status();
+}
+
+// ---- out[r, c] = src[r, c] with row strides: a tensor into a band of columns of a wider one ------
+template <typename T>
+__global__ void copy_columns_kernel(const T* __restrict__ src, long long src_stride, T* __restrict__ out,
+                                    long long out_stride, int rows, int cols) {
+    for (int r = blockIdx.y; r < rows; r += gridDim.y) {
+        const T* s = src + r * src_stride;
+        T* o = out + r * out_stride;
+        for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x) o[c] = s[c];
+    }
+}
+
+WLLM_API int wllm_copy_columns(const void* src, long long src_stride, void* out, long long out_stride, int is_bf16,
+                               int rows, int cols, hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return 0;
+    const dim3 grid(cols < 4096 ? (cols + 255) / 256 : 16, rows < 16384 ? rows : 16384);
+    if (is_bf16)
+        copy_columns_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(src), src_stride, static_cast<bf16*>(out),
+                                                            out_stride, rows, cols);
+    else
+        copy_columns_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(src), src_stride,
+                                                             static_cast<float*>(out), out_stride, rows, cols);
+    return launch_status();
+}
+
+// ---- the residual stream takes what is pending and one more addend, in float32:
+// x = ((x + delta) + bias) + addend, with delta a tensor of the activation type or a stack of float32
+// partial sums added in stack order, bias a row, addend a tensor of x's shape; each may be absent ----
+template <typename TD>
+__global__ void stream_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits, size_t split_stride,
+                                  const float* __restrict__ bias, const float* __restrict__ addend, long long total,
+                                  int hidden) {
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+        float v = x[i];
+        if (delta) {
+            if (sizeof(TD) == sizeof(float) && splits > 1)
+                v += stack_sum(reinterpret_cast<const float*>(delta) + i, splits, split_stride);
+            else
+                v += to_float(delta[i]);
+        }
+        if (bias) v += bias[i % hidden];
+        if (addend) v += addend[i];
+        x[i] = v;
+    }
+}
+
+WLLM_API int wllm_stream_add(float* x, const void* delta, int delta_bf16, int splits, long long split_stride,
+                             const float* bias, const float* addend, int rows, int hidden, hipStream_t stream) {
+    const long long total = static_cast<long long>(rows) * hidden;
+    if (total <= 0) return 0;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (delta_bf16)
+        stream_add_kernel<bf16><<<static_cast<int>(blocks), 256, 0, stream>>>(
+            x, static_cast<const bf16*>(delta), splits, static_cast<size_t>(split_stride), bias, addend, total, hidden);
+    else
+        stream_add_kernel<float><<<static_cast<int>(blocks), 256, 0, stream>>>(
+            x, static_cast<const float*>(delta), splits, static_cast<size_t>(split_stride), bias, addend, total, hidden);
+    return launch_status();
+}

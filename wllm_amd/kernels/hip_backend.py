@@ -32,8 +32,8 @@ _SIGNATURES = {
     "wllm_gemm_residual": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_qkv_rope": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
                       c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                      c_float, c_float, c_void_p],
+    "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                      c_int, c_float, c_float, c_void_p],
     "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -42,19 +42,20 @@ _SIGNATURES = {
     "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                     c_float, c_int, c_void_p],
+                                     c_float, c_int, c_int, c_float, c_void_p],
     "wllm_paged_attention_generic_chunk_keys": [],
     "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                  c_int, c_void_p],
+                                  c_int, c_int, c_float, c_void_p],
     "wllm_paged_attention_mfma_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
-                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                      c_float, c_void_p],
     "wllm_paged_attention_prefill_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                         c_void_p],
+                                         c_int, c_float, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                     c_void_p],
+                                     c_int, c_float, c_void_p],
     "wllm_gemm_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_split_sum": [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -122,14 +123,14 @@ class HipBackend:
         self._on_gpu(*[a for a in list(args) + list(kwargs.values()) if isinstance(a, torch.Tensor)])
         self._check(op.launch(fn[1], self._stream(), *args, **kwargs), op.name)
 
-    def rms_norm(self, x, weight, eps, offset, out, delta, rows):
-        self._on_gpu(x, weight, out, delta, rows)
+    def rms_norm(self, x, weight, eps, offset, out, delta, rows, delta_bias=None):
+        self._on_gpu(x, weight, out, delta, rows, delta_bias)
         splits, stride = 1, 0
         if delta is not None and delta.dim() == 3:
             splits, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
         self._check(self.lib.wllm_rms_norm(
             _ptr(x), _ptr(delta), int(delta is not None and delta.dtype == torch.bfloat16), splits, stride,
-            _ptr(weight), _ptr(rows), _ptr(out), int(out.dtype == torch.bfloat16), out.shape[0], x.shape[1], eps,
+            _ptr(delta_bias), _ptr(weight), _ptr(rows), _ptr(out), int(out.dtype == torch.bfloat16), out.shape[0], x.shape[1], eps,
             offset, self._stream()), "rms_norm")
 
     def rope_and_cache_write(self, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
@@ -233,8 +234,9 @@ class HipBackend:
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
-                        plan=None):
+                        plan=None, softcap=0.0):
         self._on_gpu(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out)
+        q_stride = qkv.shape[1]         # a row begins with the query heads; this many elements lie between two rows
         if plan is not None:
             if not self.mfma_attention_takes(qkv.dtype, head_dim, page_size):
                 raise KernelError("paged_attention: a plan was given for sizes the matrix-core kernel does not take")
@@ -244,7 +246,7 @@ class HipBackend:
                         _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.prefill_items), plan.num_prefill,
                         plan.prefill_rows, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
                         _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                        block_tables.shape[1], scale, window, self._stream()),
+                        block_tables.shape[1], scale, window, q_stride, softcap, self._stream()),
                         "paged_attention (prompt portions, matrix cores, float32)")
                 if plan.num_items == 0 and plan.num_reduce == 0:
                     return
@@ -252,7 +254,7 @@ class HipBackend:
                     _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), _ptr(plan.live_items), plan.num_items,
                     _ptr(plan.reduce_items), plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(out),
                     _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                    block_tables.shape[1], scale, window, self._stream()), "paged_attention (matrix cores, float32)")
+                    block_tables.shape[1], scale, window, q_stride, softcap, self._stream()), "paged_attention (matrix cores, float32)")
                 return
             if plan.num_prefill:
                 self._check(self.lib.wllm_paged_attention_prefill(
@@ -260,7 +262,7 @@ class HipBackend:
                     plan.prefill_rows,
                     _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(plan.partial_o),
                     _ptr(plan.partial_ml), num_heads, num_kv_heads,
-                    head_dim, page_size, block_tables.shape[1], scale, window, self._stream()),
+                    head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, self._stream()),
                     "paged_attention (prompt portions, matrix cores)")
             if plan.num_items == 0 and plan.num_reduce == 0:
                 return
@@ -269,7 +271,7 @@ class HipBackend:
                 _ptr(plan.live_items), plan.num_items, _ptr(plan.reduce_items),
                 plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
                 _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                block_tables.shape[1], scale, window, self._stream()), "paged_attention (matrix cores)")
+                block_tables.shape[1], scale, window, q_stride, softcap, self._stream()), "paged_attention (matrix cores)")
             return
         if head_dim % 4 or head_dim > 256:
             raise KernelError(f"paged_attention: head_dim {head_dim} is not a multiple of 4 up to 256")
@@ -291,7 +293,7 @@ class HipBackend:
             _ptr(qkv), _ptr(cache), int(qkv.dtype == torch.bfloat16), _ptr(block_tables), _ptr(token_segment),
             _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(self._generic_partial_o),
             _ptr(partial_ml), partial_tokens, max_ctx_len, qkv.shape[0], num_heads, num_kv_heads,
-            head_dim, page_size, block_tables.shape[1], scale, window, self._stream()), "paged_attention")
+            head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, self._stream()), "paged_attention")
 
     @staticmethod
     def skinny_split(n: int, k: int) -> int:
@@ -460,6 +462,13 @@ class HipBackend:
             _ptr(x), _ptr(weight), _ptr(tiles) if x.dtype == torch.float32 else c_void_p(0), int(x.dtype == torch.bfloat16),
             _ptr(out), int(out.dtype == torch.bfloat16),
             _ptr(partial), m, n, x.shape[1], self._stream()), "linear")
+
+    def gated_linear_writes_band(self, rows: int, dtype, in_features: int) -> bool:
+        """True where `gated_linear` runs the product and the activation as two kernels: the second
+        writes rows of any stride."""
+        if self.skinny_takes(dtype, rows, in_features) and in_features % 64 == 0:
+            return False
+        return not (dtype == torch.bfloat16 and 64 < rows <= self.TILE_GATED_MAX_ROWS and in_features % 64 == 0)
 
     def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
         self._on_gpu(x, weight, out, scratch, tiles)

@@ -142,12 +142,14 @@ def feed_tokens(ids: torch.Tensor, dst: torch.Tensor, src: torch.Tensor, source:
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, out: torch.Tensor,
-             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> None:
+             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+             delta_bias: Optional[torch.Tensor] = None) -> None:
     """out = x * rsqrt(mean(x^2) + eps) * (offset + weight), all in float32, cast to out's dtype.
 
     x float32 [n, H]; weight float32 [H]; out T [m, H].  With `delta` (T [n, H], or a stack
     float32 [S, n, H] of partial sums that are added in order) the row normalised is
-    x + delta.  Without `rows`, m = n and the sum is written back
+    x + delta; `delta_bias` (float32 [H]) is a row added to every row with it (the bias of the
+    projection that made delta).  Without `rows`, m = n and the sum is written back
     to x (the residual stream moves on).  With `rows` (int32 [m]) only those rows are
     read, x is left alone and out[i] belongs to row rows[i].
     """
@@ -167,8 +169,13 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, o
         _need(rows.dim() == 1, "rows: expected one axis")
         m = rows.shape[0]
     _dense(out, "out", _ACT, (m, h))
+    if delta_bias is not None:
+        _dense(delta_bias, "delta_bias", torch.float32, (h,))
     if m:
-        backend().rms_norm(x, weight, float(eps), float(offset), out, delta, rows)
+        if delta_bias is not None:
+            backend().rms_norm(x, weight, float(eps), float(offset), out, delta, rows, delta_bias)
+        else:
+            backend().rms_norm(x, weight, float(eps), float(offset), out, delta, rows)
 
 
 def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
@@ -296,24 +303,28 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
                     token_segment: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
                     seg_ctx_len: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                     head_dim: int, page_size: int, scale: float, window: int = 0,
-                    max_q_len: int = 0, max_ctx_len: int = 0, plan=None) -> None:
+                    max_q_len: int = 0, max_ctx_len: int = 0, plan=None, softcap: float = 0.0) -> None:
     """Softmax attention of every query over the keys of its own request in the paged cache.
 
     The batch is a row of segments; segment s holds tokens seg_q_start[s] .. +seg_q_len[s],
     the last seg_q_len[s] positions of a request that is seg_ctx_len[s] long after this
     step.  Token i of it is at position p = ctx_len - q_len + i and sees keys
     max(0, p - window + 1) .. p (window 0: from key 0).  Query head h uses key/value head
-    h // (num_heads // num_kv_heads).  Scores are scaled by `scale`; scores, softmax and the
-    weighted sum accumulate in float32.  qkv as in `rope_and_cache_write` (only the queries
-    are read); block_tables int32 [S, max_pages]; out T [n, num_heads*head_dim].
+    h // (num_heads // num_kv_heads).  Scores are scaled by `scale` and then, with `softcap` c > 0,
+    bent to c * tanh(score / c); scores, softmax and the weighted sum accumulate in float32.
+    qkv T [n, width]: a row begins with the num_heads query heads, which is all that is read of it
+    (the row of `rope_and_cache_write`, or any wider one); block_tables int32 [S, max_pages];
+    out T [n, num_heads*head_dim].
     max_q_len / max_ctx_len are host-side bounds of the segment arrays (0: unknown).
     `plan`: what `plan_paged_attention` returned for these segments and sizes, or None.
     """
-    width = (num_heads + 2 * num_kv_heads) * head_dim
+    width = num_heads * head_dim
     _dense(qkv, "qkv", _ACT)
-    _need(qkv.dim() == 2 and qkv.shape[1] == width, lambda: f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
+    _need(qkv.dim() == 2 and qkv.shape[1] >= width and qkv.shape[1] % 8 == 0,
+          lambda: f"qkv: shape {tuple(qkv.shape)}, expected [n, at least {width} and a multiple of 8]")
     n = qkv.shape[0]
     _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
+    _need(softcap >= 0.0, "softcap must not be negative (0: none)")
     _dense(cache, "cache", qkv.dtype)
     _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
           lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
@@ -328,7 +339,102 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     if n:
         backend().paged_attention(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len,
                                   out, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
-                                  int(max_q_len), int(max_ctx_len), plan)
+                                  int(max_q_len), int(max_ctx_len), plan, **({"softcap": float(softcap)} if softcap else {}))
+
+
+def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                 inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], *,
+                 num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, interleaved: bool = False,
+                 norm_eps: Optional[float] = None, values_are_keys: bool = False,
+                 parts: Optional[torch.Tensor] = None) -> None:
+    """What `rope_and_cache_write` does, for attention blocks that do more between projection and
+    attention.  rows T [n, width]: num_heads query heads, num_kv_heads key heads, num_kv_heads value
+    heads unless `values_are_keys`, then any further columns.  In this order, in float32: every
+    element takes its bias (float32 [width] or None) and, with `parts` (float32 [S, n, width]), is
+    the sum of the stack in order instead of what the row held; with `values_are_keys` a key head
+    as it is now is stored as the value head; the first 2 * len(inv_freq) elements of every query
+    and key head turn by position * inv_freq[j], pair j being elements (2j, 2j + 1) if
+    `interleaved`, else (j, j + len(inv_freq)); with `norm_eps` every query and key head is
+    divided by sqrt(mean of its squares + norm_eps); the heads are written back and the key heads
+    stored.  slots, cache as in `rope_and_cache_write` (both None: nothing is stored)."""
+    heads = num_heads + (1 if values_are_keys else 2) * num_kv_heads
+    _dense(rows, "rows", _ACT)
+    _need(rows.dim() == 2 and rows.shape[1] >= heads * head_dim,
+          lambda: f"rows: shape {tuple(rows.shape)}, expected [n, at least {heads * head_dim}]")
+    n, width = rows.shape
+    _need(0 < head_dim <= 256, "head_dim: at most 256")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, (width,))
+    if parts is not None:
+        _need(parts.dim() == 3 and parts.shape[0] >= 1, "parts: expected [S, n, width]")
+        _dense(parts, "parts", torch.float32, (parts.shape[0], n, width))
+    _dense(positions, "positions", torch.int32, (n,))
+    if inv_freq is not None:
+        _dense(inv_freq, "inv_freq", torch.float32)
+        _need(inv_freq.dim() == 1 and 0 < 2 * inv_freq.shape[0] <= head_dim,
+              lambda: f"inv_freq: {tuple(inv_freq.shape)} does not fit head_dim {head_dim}")
+    _need(norm_eps is None or norm_eps >= 0.0, "norm_eps must not be negative")
+    _need((slots is None) == (cache is None), "slots and cache go together")
+    if cache is not None:
+        _dense(slots, "slots", torch.int32, (n,))
+        _dense(cache, "cache", rows.dtype)
+        _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
+              lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+    if n:
+        call("head_prepare", rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
+             page_size, bool(interleaved), norm_eps, bool(values_are_keys), parts)
+
+
+def _band(t: torch.Tensor, name: str, dtype, rows: int, cols: int) -> None:
+    """A tensor [rows, cols] or a band of columns of a wider contiguous one."""
+    if not isinstance(t, torch.Tensor) or t.dtype != dtype:
+        raise KernelShapeError(f"{name}: expected a tensor of {dtype}")
+    _need(t.dim() == 2 and tuple(t.shape) == (rows, cols), lambda: f"{name}: shape {tuple(t.shape)}, expected {(rows, cols)}")
+    _need(rows == 0 or cols == 0 or (t.stride(1) == 1 and t.stride(0) >= cols),
+          lambda: f"{name}: strides {t.stride()}: rows must be runs of consecutive elements")
+
+
+def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> None:
+    """out = a * sigmoid(gate), in float32, cast to T.  All T [n, c]; each may be a band of columns
+    of a wider tensor (a view whose rows are runs of consecutive elements); out may be a."""
+    _need(a.dim() == 2 and a.dtype in _ACT, "a: expected T [n, c]")
+    n, c = a.shape
+    for t, name in ((a, "a"), (gate, "gate"), (out, "out")):
+        _band(t, name, a.dtype, n, c)
+    if n and c:
+        call("sigmoid_gate", a, gate, out)
+
+
+def copy_columns(src: torch.Tensor, out: torch.Tensor) -> None:
+    """out = src; both T [n, c], each possibly a band of columns of a wider tensor."""
+    _need(src.dim() == 2 and src.dtype in _ACT, "src: expected T [n, c]")
+    n, c = src.shape
+    _band(src, "src", src.dtype, n, c)
+    _band(out, "out", src.dtype, n, c)
+    if n and c:
+        call("copy_columns", src, out)
+
+
+def stream_add(x: torch.Tensor, addend: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
+               delta_bias: Optional[torch.Tensor] = None) -> None:
+    """x = ((x + delta) + delta_bias) + addend in float32, in place.  x float32 [n, H]; delta T [n, H]
+    or a stack float32 [S, n, H] added in order; delta_bias float32 [H]; addend float32 [n, H]; any
+    of the three may be None."""
+    _dense(x, "x", torch.float32)
+    _need(x.dim() == 2, "x: expected [tokens, hidden]")
+    n, h = x.shape
+    if delta is not None:
+        if delta.dim() == 3:
+            _dense(delta, "delta", torch.float32, (delta.shape[0], n, h))
+            _need(delta.shape[0] >= 1, "delta: an empty stack")
+        else:
+            _dense(delta, "delta", _ACT, (n, h))
+    if delta_bias is not None:
+        _dense(delta_bias, "delta_bias", torch.float32, (h,))
+    if addend is not None:
+        _dense(addend, "addend", torch.float32, (n, h))
+    if n and (delta is not None or delta_bias is not None or addend is not None):
+        call("stream_add", x, addend, delta, delta_bias)
 
 
 def plan_paged_attention(host_q_len, host_ctx_len, *, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -438,11 +544,12 @@ ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
 
 
 def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> None:
-    """out = act(gate_up[:, :I]) * gate_up[:, I:], in float32, cast to T.  gate_up T [n, 2I]."""
+    """out = act(gate_up[:, :I]) * gate_up[:, I:], in float32, cast to T.  gate_up T [n, 2I]; out T [n, I],
+    possibly a band of columns of a wider tensor."""
     _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
     _dense(gate_up, "gate_up", _ACT)
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate_up: expected [n, 2*intermediate]")
-    _dense(out, "out", gate_up.dtype, (gate_up.shape[0], gate_up.shape[1] // 2))
+    _band(out, "out", gate_up.dtype, gate_up.shape[0], gate_up.shape[1] // 2)
     if gate_up.shape[0]:
         call("gated_activation", gate_up, out, activation)
 
@@ -475,10 +582,17 @@ def gated_linear_norm_takes(rows: int, dtype: torch.dtype, in_features: int) -> 
     return bool(backend().gated_linear_norm_takes(rows, dtype, in_features))
 
 
+def gated_linear_writes_band(rows: int, dtype: torch.dtype, in_features: int) -> bool:
+    """Whether `gated_linear` at these sizes can write `out` as a band of columns of a wider tensor (it
+    can where the product and the activation are two kernels)."""
+    return bool(getattr(backend(), "gated_linear_writes_band", lambda *a: False)(rows, dtype, in_features))
+
+
 def gated_linear(x, weight: torch.Tensor, out: torch.Tensor, activation: str,
                  scratch: Optional[torch.Tensor], tiles: Optional[torch.Tensor] = None) -> None:
     """out = act(x @ Wg^T) * (x @ Wu^T) with weight = [Wg; Wu] stacked, T [2I, k]; x T [m, k];
-    out T [m, I]; scratch T [m, 2I] may be used for the unfused product.  `tiles` is
+    out T [m, I] (a band of a wider tensor where `gated_linear_writes_band`); scratch T [m, 2I] may be
+    used for the unfused product.  `tiles` is
     `tile_weight(weight, halves=2)`.  x may be a `NormOnLoad` where `gated_linear_norm_takes` says so:
     the norm is then applied as the kernel reads the residual stream (scratch is not used)."""
     _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
@@ -498,7 +612,11 @@ def gated_linear(x, weight: torch.Tensor, out: torch.Tensor, activation: str,
     _need(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.shape[0] % 2 == 0,
           lambda: f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
     inter = weight.shape[0] // 2
-    _dense(out, "out", x.dtype, (x.shape[0], inter))
+    if out.is_contiguous():
+        _dense(out, "out", x.dtype, (x.shape[0], inter))
+    else:
+        _band(out, "out", x.dtype, x.shape[0], inter)
+        _need(gated_linear_writes_band(x.shape[0], x.dtype, x.shape[1]), "out: a band of columns at sizes whose kernel writes whole rows")
     _dense(scratch, "scratch", x.dtype, (x.shape[0], 2 * inter))
     _check_tiles(tiles, weight, 2)
     if x.shape[0]:
@@ -547,7 +665,7 @@ def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
 
 # ---- the framework's own operations that go through the same door as a part's ------------------
 def _register_own() -> None:
-    from ctypes import c_float, c_int, c_void_p
+    from ctypes import c_float, c_int, c_longlong, c_void_p
     p = pointer
     register_op("embed_lookup", entry_point="wllm_embed_lookup",
                 argtypes=[c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -559,10 +677,46 @@ def _register_own() -> None:
                 launch=lambda fn, stream, ids, dst, src, source: fn(
                     p(ids), p(dst), p(src), p(source), dst.shape[0], ids.shape[0], source.shape[0], stream))
     register_op("gated_activation", entry_point="wllm_gated_activation",
-                argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_longlong, c_void_p],
                 launch=lambda fn, stream, gate_up, out, activation: fn(
                     p(gate_up), p(out), int(gate_up.dtype == torch.bfloat16), ACTIVATIONS[activation], gate_up.shape[0],
-                    out.shape[1], stream))
+                    out.shape[1], out.stride(0) if out.shape[0] > 1 else out.shape[1], stream))
+
+
+    def prepare(fn, stream, rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
+                page_size, interleaved, norm_eps, values_are_keys, parts):
+        splits, stride = (parts.shape[0], parts.shape[1] * parts.shape[2]) if parts is not None else (0, 0)
+        return fn(p(rows), int(rows.dtype == torch.bfloat16), rows.shape[1], p(parts), splits, stride, p(bias),
+                  p(positions), p(inv_freq), p(slots), p(cache), cache.shape[0] if cache is not None else 0,
+                  rows.shape[0], num_heads, num_kv_heads, head_dim,
+                  2 * inv_freq.shape[0] if inv_freq is not None else 0, int(interleaved),
+                  float(norm_eps) if norm_eps is not None else -1.0, int(values_are_keys), page_size, stream)
+
+    register_op("head_prepare", entry_point="wllm_head_prepare",
+                argtypes=[c_void_p, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                launch=prepare)
+    register_op("sigmoid_gate", entry_point="wllm_sigmoid_gate",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, a, gate, out: fn(
+                    p(a), a.stride(0), p(gate), gate.stride(0), p(out), out.stride(0), int(a.dtype == torch.bfloat16),
+                    a.shape[0], a.shape[1], stream))
+    register_op("copy_columns", entry_point="wllm_copy_columns",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, src, out: fn(
+                    p(src), src.stride(0), p(out), out.stride(0), int(src.dtype == torch.bfloat16), src.shape[0],
+                    src.shape[1], stream))
+
+    def add(fn, stream, x, addend, delta, delta_bias):
+        splits, stride = 1, 0
+        if delta is not None and delta.dim() == 3:
+            splits, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+        return fn(p(x), p(delta), int(delta is not None and delta.dtype == torch.bfloat16), splits, stride,
+                  p(delta_bias), p(addend), x.shape[0], x.shape[1], stream)
+
+    register_op("stream_add", entry_point="wllm_stream_add",
+                argtypes=[c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_int, c_int, c_void_p],
+                launch=add)
 
 
 _register_own()

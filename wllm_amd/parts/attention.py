@@ -8,6 +8,13 @@ being a segment of one.  Head h of the q/k/v rows is columns h*head_dim ..
 (h+1)*head_dim of the projection (llama.py:103-105).  The three projection
 matrices are stacked at load so that one product makes the [n, (nh+2nkv)*d]
 row the kernels read.
+
+The specification's options widen the row and the steps between projection and attention
+(`ops.head_prepare` then stands where `ops.rope_and_cache_write` stands for the plain form): a
+rotation of interleaved pairs or of a part of the head, a unit norm of queries and keys, values
+that are the keys as projected (the row has no value heads), a cap on the scores, and an output
+gate whose projection is stacked behind the heads (row: queries, keys, [values], [gate]) and
+multiplied into the attention's result before the output projection, which may have a bias.
 """
 from __future__ import annotations
 
@@ -35,16 +42,33 @@ class PagedAttention:
         if spec.head_dim % ops.HEAD_DIM_STEP or not 0 < spec.head_dim <= ops.MAX_HEAD_DIM:
             raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of "
                              f"{ops.HEAD_DIM_STEP} up to {ops.MAX_HEAD_DIM}")
+        if spec.values_are_keys and (spec.v_weight or spec.v_bias):
+            raise ValueError("values_are_keys: there is no value projection to name")
+        if spec.softcap is not None and not spec.softcap > 0:
+            raise ValueError(f"softcap must be positive or None, got {spec.softcap}")
+        if spec.qk_norm_eps is not None and spec.qk_norm_eps < 0:
+            raise ValueError(f"qk_norm_eps must not be negative, got {spec.qk_norm_eps}")
         self.spec = spec
         self.position = build_position(spec.position)
         self.w_qkv = None
         self.b_qkv = None
         self.w_o = None
+        self.b_o = None
+        # the plain form runs the kernels that were written for it; anything else the general ones
+        self.plain = not (spec.softcap or spec.qk_norm_eps is not None or spec.values_are_keys or spec.gate_weight
+                          or getattr(self.position, "interleaved", False))
 
     @property
     def qkv_width(self) -> int:
+        """Columns of the projected row: queries, keys, values (unless they are the keys), gate."""
         s = self.spec
-        return (s.num_heads + 2 * s.num_kv_heads) * s.head_dim
+        heads = s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads + (s.num_heads if s.gate_weight else 0)
+        return heads * s.head_dim
+
+    @property
+    def gate_offset(self) -> int:
+        s = self.spec
+        return (s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads) * s.head_dim
 
     def expected_tensors(self) -> dict:
         s = self.spec
@@ -52,10 +76,13 @@ class PagedAttention:
         out = {
             s.q_weight: ExpectedTensor((q, s.hidden_size)),
             s.k_weight: ExpectedTensor((kv, s.hidden_size)),
-            s.v_weight: ExpectedTensor((kv, s.hidden_size)),
             s.o_weight: ExpectedTensor((s.hidden_size, q)),
         }
-        for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv)):
+        if not s.values_are_keys:
+            out[s.v_weight] = ExpectedTensor((kv, s.hidden_size))
+        if s.gate_weight:
+            out[s.gate_weight] = ExpectedTensor((q, s.hidden_size))
+        for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv), (s.o_bias, s.hidden_size)):
             if name is not None:
                 out[name] = ExpectedTensor((width,), role="vector")
         if hasattr(self.position, "expected_tensors"):      # a position encoding with tensors of its own
@@ -64,13 +91,18 @@ class PagedAttention:
 
     def load(self, fetch) -> None:
         s = self.spec
-        w = torch.cat([fetch.matrix(s.q_weight), fetch.matrix(s.k_weight), fetch.matrix(s.v_weight)], dim=0)
+        names = [s.q_weight, s.k_weight] + ([] if s.values_are_keys else [s.v_weight]) + ([s.gate_weight] if s.gate_weight else [])
+        w = torch.cat([fetch.matrix(name) for name in names], dim=0)
         self.w_qkv, self.t_qkv = load_matrix(fetch, w)        # the matrix and its tile-major copy
         self.w_o, self.t_o = load_matrix(fetch, fetch.matrix(s.o_weight))
+        if s.o_bias is not None:
+            self.b_o = fetch.to_device(fetch.vector(s.o_bias))
         if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
             q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
-            parts = [fetch.vector(name) if name is not None else torch.zeros(width)
-                     for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv))]
+            biases = [(s.q_bias, q), (s.k_bias, kv)] + ([] if s.values_are_keys else [(s.v_bias, kv)])
+            parts = [fetch.vector(name) if name is not None else torch.zeros(width) for name, width in biases]
+            if s.gate_weight:
+                parts.append(torch.zeros(q))
             self.b_qkv = fetch.to_device(torch.cat(parts))
         if hasattr(self.position, "load"):
             self.position.load(fetch)
@@ -92,6 +124,7 @@ class PagedAttention:
         """The step's work items for attention of this shape: made once a step, shared by all
         layers of the shape; of fixed shape and rewritten in place in a captured graph."""
         s = self.spec
+        # (the plan depends on these alone: layers that differ in their rows' width or cap share it)
         shape = dict(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=page_size,
                      window=s.window or 0)
 
@@ -106,7 +139,10 @@ class PagedAttention:
 
         return ctx.plan(("attention",) + tuple(shape.values()), build, refresh)
 
-    def forward(self, ctx, entry: int, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx, entry: int, h: torch.Tensor, product_input: Optional[torch.Tensor] = None):
+        """`product_input`: a band of columns [n, heads * head_dim] of a wider buffer into which the
+        input of the output projection is to be written (a block that makes one product of several
+        parts' last products asks for it); the returned `Product` then names that band."""
         s = self.spec
         n = h.shape[0]
         qkv = ctx.buffer("qkv", (n, self.qkv_width), h.dtype)
@@ -118,7 +154,16 @@ class PagedAttention:
         inv_freq = self.position.inv_freq
         apply = getattr(self.position, "apply", None)
         rotary_dim = 2 * inv_freq.shape[0] if inv_freq is not None else s.head_dim
-        if apply is not None:
+        if not self.plain:
+            if apply is not None:
+                raise NotImplementedError("a position encoding with a step of its own beside the attention's options")
+            projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
+            ops.head_prepare(
+                qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage, num_heads=s.num_heads,
+                num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
+                interleaved=getattr(self.position, "interleaved", False), norm_eps=s.qk_norm_eps,
+                values_are_keys=s.values_are_keys, parts=projected if projected.dim() == 3 else None)
+        elif apply is not None:
             ops.linear(h, self.w_qkv, qkv, self.t_qkv)
             if self.b_qkv is not None:
                 qkv += self.b_qkv.to(qkv.dtype)
@@ -145,6 +190,15 @@ class PagedAttention:
             ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
-            plan=self._work_items(ctx, pages.page_size))
+            plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0)
+        if s.gate_weight:
+            # the gate's columns lie behind the heads in the projected row
+            gate = qkv[:, self.gate_offset:self.gate_offset + s.num_heads * s.head_dim]
+            target = product_input if product_input is not None else attn
+            ops.sigmoid_gate(attn, gate, target)
+            attn = target
+        elif product_input is not None:
+            ops.copy_columns(attn, product_input)
+            attn = product_input
         # the stream adds the output projection: at once, or through the next norm, partial sums and all
-        return Product("mixer_out", attn, self.w_o, self.t_o)
+        return Product("mixer_out", attn, self.w_o, self.t_o, bias=self.b_o)

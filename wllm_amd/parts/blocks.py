@@ -6,6 +6,13 @@ A part's contribution is not added at once: it is left pending on the stream and
 the next norm kernel adds it while it normalises, so the sum is formed in
 float32 and the stream is read and written once per norm.  In a decode step of few
 rows the norm kernel can fall away altogether (`ResidualStream`).
+
+"parallel": h = norm(x); x += mixer(h) + feed_forward(h).  One norm, both parts read its
+output.  Both parts end in a product (attention's output projection, the feed-forward's down
+projection), and the sum of two products is one product over the two inputs side by side:
+[a | f] [Wo | Wd]^T.  The block lays the two weights side by side at load, lets the parts write
+their products' inputs into the two bands of one buffer, and makes that one product: the sum is
+formed in the product's float32 accumulators, and the stream sees one contribution.
 """
 from __future__ import annotations
 
@@ -32,31 +39,44 @@ class ResidualStream:
     def __init__(self, x: torch.Tensor, pending: Optional[torch.Tensor] = None):
         self.x = x
         self.pending = pending
+        self.pending_bias: Optional[torch.Tensor] = None      # float32 [H]: a row that comes with `pending`
         self.sumsq: Optional[torch.Tensor] = None      # float32 [n, bands]: sums of squares of x as it is now
 
     def normed(self, norm, out: torch.Tensor, rows=None) -> torch.Tensor:
         """norm(x + pending).  Without `rows` the sum becomes the new x."""
-        norm.forward(self.x, out, delta=self.pending, rows=rows)
-        if rows is None and self.pending is not None:
-            self.pending = None
+        if self.pending_bias is not None:
+            norm.forward(self.x, out, delta=self.pending, rows=rows, delta_bias=self.pending_bias)
+        else:
+            norm.forward(self.x, out, delta=self.pending, rows=rows)
+        if rows is None and (self.pending is not None or self.pending_bias is not None):
+            self.pending = self.pending_bias = None
             self.sumsq = None
         return out
+
+    def settle(self, addend: Optional[torch.Tensor] = None) -> None:
+        """x takes what is pending, and `addend` (float32, x's shape) with it, without a norm."""
+        if self.pending is None and self.pending_bias is None and addend is None:
+            return
+        ops.stream_add(self.x, addend, self.pending, self.pending_bias)
+        self.pending = self.pending_bias = None
+        self.sumsq = None
 
     def input_for(self, ctx, norm, part):
         """What `part` gets as its input: the normalised stream as a tensor, or, where the part and
         the norm allow it, the recipe to normalise it while reading (`ops.NormOnLoad`)."""
         n, hidden = self.x.shape
-        if (self.pending is None and self.sumsq is not None and hasattr(norm, "on_load")
+        if (self.pending is None and self.pending_bias is None and self.sumsq is not None and hasattr(norm, "on_load")
                 and getattr(part, "takes_norm_on_load", lambda *a: False)(n, ctx.dtype)):
             return norm.on_load(self.x, self.sumsq, ctx.dtype)
         return self.normed(norm, ctx.buffer("normed", (n, hidden), ctx.dtype))
 
     def add(self, ctx, y) -> None:
-        if self.pending is not None:
+        if self.pending is not None or self.pending_bias is not None:
             raise RuntimeError("a contribution is already pending; normalise before adding another")
         if isinstance(y, Product):
             n, hidden = self.x.shape
-            if ops.linear_residual_takes(n, y.x.dtype, hidden, y.x.shape[1]):
+            self.pending_bias = y.bias
+            if y.bias is None and y.x.is_contiguous() and ops.linear_residual_takes(n, y.x.dtype, hidden, y.x.shape[1]):
                 sumsq = ctx.buffer("sumsq", ops.linear_residual_sumsq_shape(n, hidden), torch.float32)
                 ops.linear_residual(y.x, y.weight, self.x, sumsq, y.tiles)
                 self.sumsq = sumsq
@@ -82,3 +102,55 @@ class PreNormBlock:
         stream.add(ctx, self.mixer.forward(ctx, entry, h))
         h = stream.input_for(ctx, self.feed_forward_norm, self.feed_forward)
         stream.add(ctx, self.feed_forward.forward(ctx, h))
+
+
+@register_block("parallel")
+class ParallelBlock:
+    """x += mixer(h) + feed_forward(h) with h = norm(x), as one product over both parts' inputs."""
+
+    def __init__(self, spec: BlockSpec):
+        if spec.feed_forward_norm is not None:
+            raise ValueError("a parallel block has one norm; feed_forward_norm must be None")
+        self.spec = spec
+        self.mixer = build_mixer(spec.mixer)
+        self.feed_forward = build_feed_forward(spec.feed_forward) if spec.feed_forward is not None else None
+        self.mixer_norm = build_norm(spec.mixer_norm)
+        self.w_joint = self.t_joint = None      # [Wo | Wd] and its tile-major copy, once loaded
+        self.k_mixer = self.k_ff = 0
+
+    def parts(self) -> list:
+        own = [self.mixer_norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+        return own + [self]         # the block itself loads last: it joins what its parts loaded
+
+    def expected_tensors(self) -> dict:
+        return {}
+
+    def load(self, fetch) -> None:
+        """Lays the two last weights side by side, [Wo | Wd], for the one product of `forward`, and
+        lets go of the parts' own copies.  Parts whose last product is not a plain attribute pair
+        (`w_o`/`w_down`) keep theirs, and the block adds the two products one after the other."""
+        m, f = self.mixer, self.feed_forward
+        if f is None or getattr(m, "w_o", None) is None or getattr(f, "w_down", None) is None:
+            return
+        self.k_mixer, self.k_ff = m.w_o.shape[1], f.w_down.shape[1]
+        self.w_joint = torch.cat([m.w_o, f.w_down], dim=1).contiguous()
+        self.t_joint = ops.tile_weight(self.w_joint) if getattr(fetch, "tiled_copies", False) else None
+        m.w_o = m.t_o = f.w_down = f.t_down = None
+
+    def forward(self, ctx, entry: int, stream: ResidualStream) -> None:
+        n, hidden = stream.x.shape
+        h = stream.normed(self.mixer_norm, ctx.buffer("normed", (n, hidden), ctx.dtype))
+        if self.feed_forward is None:
+            stream.add(ctx, self.mixer.forward(ctx, entry, h))
+            return
+        if self.w_joint is None:
+            # two products, one after the other: the second waits as the stream's pending contribution
+            stream.add(ctx, self.mixer.forward(ctx, entry, h))
+            stream.settle()
+            stream.add(ctx, self.feed_forward.forward(ctx, h))
+            return
+        both = ctx.buffer("joint_in", (n, self.k_mixer + self.k_ff), ctx.dtype)
+        a = self.mixer.forward(ctx, entry, h, product_input=both[:, :self.k_mixer])
+        f = self.feed_forward.forward(ctx, h, product_input=both[:, self.k_mixer:])
+        bias = a.bias if f.bias is None else (f.bias if a.bias is None else a.bias + f.bias)
+        stream.add(ctx, Product("block_out", both, self.w_joint, self.t_joint, bias=bias))

@@ -32,8 +32,10 @@ class Product:
     also leaves what the next norm needs (`ops.linear_residual`), or as a tensor (or a stack of
     partial sums) that the next norm kernel adds."""
 
-    def __init__(self, name: str, x: torch.Tensor, weight: torch.Tensor, tiles: Optional[torch.Tensor] = None):
-        self.name, self.x, self.weight, self.tiles = name, x, weight, tiles
+    def __init__(self, name: str, x: torch.Tensor, weight: torch.Tensor, tiles: Optional[torch.Tensor] = None,
+                 bias: Optional[torch.Tensor] = None):
+        # `bias`: float32 [out], a row that belongs to the product; whoever adds the product adds it too
+        self.name, self.x, self.weight, self.tiles, self.bias = name, x, weight, tiles, bias
 
     def make(self, ctx) -> torch.Tensor:
         return project(ctx, self.name, self.x, self.weight, tiles=self.tiles)

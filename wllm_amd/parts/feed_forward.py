@@ -44,13 +44,23 @@ class GatedMLP:
         """Whether `forward` may be given `ops.NormOnLoad` instead of the normalised tensor."""
         return ops.gated_linear_norm_takes(rows, dtype, self.spec.hidden_size)
 
-    def forward(self, ctx, h):
+    def forward(self, ctx, h, product_input=None):
+        """`product_input`: a band of columns [n, intermediate] of a wider buffer into which the input
+        of the down projection is to be written (a block that makes one product of several parts'
+        last products asks for it); the returned `Product` then names that band."""
         s = self.spec
         n = h.shape[0]
-        act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
         if isinstance(h, ops.NormOnLoad):
+            act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
             ops.gated_linear(h, self.w_gate_up, act, s.activation, None, self.t_gate_up)
         else:
             gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
+            if product_input is not None and ops.gated_linear_writes_band(n, h.dtype, s.hidden_size):
+                act = product_input         # the activation kernel writes the band itself
+            else:
+                act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
             ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up, self.t_gate_up)
+        if product_input is not None and act is not product_input:
+            ops.copy_columns(act, product_input)
+            act = product_input
         return Product("ffn_out", act, self.w_down, self.t_down)

@@ -151,7 +151,14 @@ class CausalLM:
         x = ctx.buffer("residual", (n, hidden), torch.float32)
         ops.embed_lookup(ctx.token_ids, self.embed_table, self.embed_scale, x)
         stream = ResidualStream(x)
+        embedded = None
+        if any(e.adds_embedding for e in self.plan.schedule):
+            # a later run adds the embedding output again: kept, since x moves on
+            embedded = ctx.buffer("embedded", (n, hidden), torch.float32)
+            ops.embed_lookup(ctx.token_ids, self.embed_table, self.embed_scale, embedded)
         for entry, e in enumerate(self.plan.schedule):
+            if e.adds_embedding:
+                stream.settle(embedded)
             self.blocks[e.layer].forward(ctx, entry, stream)
         m = ctx.num_logit_rows
         vocab = self.plan.head.vocab_size
@@ -165,7 +172,12 @@ class CausalLM:
 
 
 def build_model(raw_config: dict) -> CausalLM:
-    entry = resolve_architecture(raw_config.get("architectures"))
+    # config.json names its model under `architectures` (a list, the first known name wins) or
+    # under `architecture` (one name)
+    names = raw_config.get("architectures")
+    if not names and isinstance(raw_config.get("architecture"), str):
+        names = [raw_config["architecture"]]
+    entry = resolve_architecture(names)
     config = entry.parse_config(raw_config)
     return CausalLM(entry.build_plan(config), config)
 

@@ -25,8 +25,9 @@ class RMSNorm:
     def load(self, fetch) -> None:
         self.weight = fetch.to_device(fetch.vector(self.spec.weight))
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, delta=None, rows=None) -> torch.Tensor:
-        ops.rms_norm(x, self.weight, self.spec.eps, self.spec.weight_offset, out, delta=delta, rows=rows)
+    def forward(self, x: torch.Tensor, out: torch.Tensor, delta=None, rows=None, delta_bias=None) -> torch.Tensor:
+        ops.rms_norm(x, self.weight, self.spec.eps, self.spec.weight_offset, out, delta=delta, rows=rows,
+                     delta_bias=delta_bias)
         return out
 
     def on_load(self, residual: torch.Tensor, sumsq: torch.Tensor, dtype: torch.dtype):

@@ -3,7 +3,10 @@ float32 exactly as the reference builds it (src/wllm/models/llama.py:52-56); the
 angle position * inv_freq[j] and its sine and cosine are computed in float32
 inside the rotation kernel (llama.py:58-62), and element j is paired with
 j + rotary_dim/2 (llama.py:47-49,65-71).  The table stays float32 in every
-mode.  "none": no rotation."""
+mode.  Two options beyond that form: `pairing="interleaved"` pairs element 2j with 2j + 1, and
+`scaling_factor` divides every frequency (linear scaling of positions); with either, the table
+is worked out in float64 and rounded once.  `rotary_dim` may be less than the head: the rest of
+a head passes unchanged.  "none": no rotation."""
 from __future__ import annotations
 
 import torch
@@ -15,8 +18,10 @@ from wllm_amd.parts.specs import PositionSpec
 @register_position("rope")
 class RotaryPosition:
     def __init__(self, spec: PositionSpec):
-        if spec.pairing != "half":
-            raise ValueError(f"rope pairing {spec.pairing!r} is not implemented; only 'half'")
+        if spec.pairing not in ("half", "interleaved"):
+            raise ValueError(f"rope pairing {spec.pairing!r} is not implemented; 'half' or 'interleaved'")
+        if not spec.scaling_factor > 0.0:
+            raise ValueError(f"scaling_factor must be positive, got {spec.scaling_factor}")
         if spec.rotary_dim <= 0 or spec.rotary_dim % 2:
             raise ValueError(f"rotary_dim must be positive and even, got {spec.rotary_dim}")
         self.spec = spec
@@ -24,8 +29,16 @@ class RotaryPosition:
 
     def prepare(self, device) -> None:
         d = self.spec.rotary_dim
-        inv = 1.0 / (self.spec.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        if self.spec.pairing == "half" and self.spec.scaling_factor == 1.0:
+            inv = 1.0 / (self.spec.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        else:
+            exact = 1.0 / (float(self.spec.theta) ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
+            inv = (exact / self.spec.scaling_factor).to(torch.float32)
         self.inv_freq = inv.to(device)
+
+    @property
+    def interleaved(self) -> bool:
+        return self.spec.pairing == "interleaved"
 
 
 @register_position("none")

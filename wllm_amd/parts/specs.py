@@ -26,12 +26,14 @@ class NormSpec:
 @dataclass(frozen=True)
 class PositionSpec:
     """How positions enter a mixer.  kind "rope": rotation of query and key by
-    angles position * theta^(-2j/rotary_dim), pairing element j with
-    j + rotary_dim/2 ("half") ; kind "none": nothing."""
+    angles position * theta^(-2j/rotary_dim) / scaling_factor, pairing element j with
+    j + rotary_dim/2 ("half") or element 2j with 2j + 1 ("interleaved"); elements of a head
+    beyond rotary_dim pass unchanged.  kind "none": nothing."""
     kind: str = "rope"
     rotary_dim: int = 0
     theta: float = 10000.0
     pairing: str = "half"
+    scaling_factor: float = 1.0     # linear scaling: every frequency is divided by it
 
 
 @dataclass(frozen=True)
@@ -45,7 +47,15 @@ class AttentionSpec(MixerSpec):
     """Softmax attention of each query over the earlier keys of its request,
     read from the paged cache.  Query head h uses key/value head
     h // (num_heads // num_kv_heads).  `window` = W limits a query at position p
-    to keys p-W+1..p; None is all keys."""
+    to keys p-W+1..p; None is all keys.
+
+    Options beyond the plain form, each off by default.  `softcap` c: the scaled score s becomes
+    c * tanh(s / c) before the softmax.  `qk_norm_eps`: after the rotation every query and key
+    head is divided by sqrt(mean of its squares + eps) (a norm without a weight).
+    `values_are_keys`: there is no value projection; a key head as projected (with its bias,
+    before rotation and norm) is also the value head.  `gate_weight`: the concatenated heads are
+    multiplied by sigmoid(W_gate h) before the output projection.  `o_bias`: a bias of the output
+    projection."""
     kind: str = "attention"
     hidden_size: int = 0
     num_heads: int = 0
@@ -61,6 +71,11 @@ class AttentionSpec(MixerSpec):
     q_bias: Optional[str] = None
     k_bias: Optional[str] = None
     v_bias: Optional[str] = None
+    softcap: Optional[float] = None
+    qk_norm_eps: Optional[float] = None
+    values_are_keys: bool = False
+    gate_weight: Optional[str] = None
+    o_bias: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -84,12 +99,14 @@ class GatedMLPSpec(FeedForwardSpec):
 @dataclass(frozen=True)
 class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms, and how they are
-    arranged around the residual stream ("pre_norm": x += mixer(norm(x));
-    x += ffn(norm(x)))."""
+    arranged around the residual stream.  "pre_norm": x += mixer(norm(x));
+    x += ffn(norm(x)).  "parallel": h = mixer_norm(x); x += mixer(h) + ffn(h): one norm, both
+    sublayers read it (`feed_forward_norm` is None, and `feed_forward` may be None: then the
+    layer is its mixer alone)."""
     mixer: MixerSpec
-    feed_forward: FeedForwardSpec
+    feed_forward: Optional[FeedForwardSpec]
     mixer_norm: NormSpec
-    feed_forward_norm: NormSpec
+    feed_forward_norm: Optional[NormSpec]
     arrangement: str = "pre_norm"
 
 
@@ -120,9 +137,12 @@ class ScheduleEntry:
     """One run of a layer.  `layer` indexes ModelPlan.layers (the same layer may
     be named by several entries: its weights are shared, each run has a cache
     of its own).  `reads_cache_of` = index of an earlier schedule entry whose
-    cache this run reads instead of writing one."""
+    cache this run reads instead of writing one.  `adds_embedding`: before this run the
+    embedding output (the stream as it was before the first run) is added to the stream, as
+    a model does that sends the stream through a span of its layers several times."""
     layer: int
     reads_cache_of: Optional[int] = None
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)
