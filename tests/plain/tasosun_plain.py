@@ -55,7 +55,7 @@ def embedding(table: torch.Tensor, tokens, scale: float) -> torch.Tensor:
 
 
 def offset_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
-    """x / sqrt(mean(x^2) + eps) * (1 + w): the weight is stored around zero."""
+    """x / sqrt(mean(x^2) + eps) * (1 + w): what is stored is the weight's distance from one."""
     return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps) * (1.0 + w)
 
 

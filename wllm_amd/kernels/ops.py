@@ -320,8 +320,8 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     """
     width = num_heads * head_dim
     _dense(qkv, "qkv", _ACT)
-    _need(qkv.dim() == 2 and qkv.shape[1] >= width and qkv.shape[1] % 8 == 0,
-          lambda: f"qkv: shape {tuple(qkv.shape)}, expected [n, at least {width} and a multiple of 8]")
+    _need(qkv.dim() == 2 and qkv.shape[1] >= width,
+          lambda: f"qkv: shape {tuple(qkv.shape)}, expected [n, at least {width}]")
     n = qkv.shape[0]
     _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
     _need(softcap >= 0.0, "softcap must not be negative (0: none)")
