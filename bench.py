@@ -45,7 +45,9 @@ def step_flops(model, tokens: int, context_before: int, logit_rows: int) -> floa
     flops = 0.0
     for e in model.plan.schedule:
         block = model.blocks[e.layer]
-        flops += block.mixer.flops(tokens, keys) + block.feed_forward.flops(tokens)
+        flops += block.mixer.flops(tokens, keys)
+        if block.feed_forward is not None:
+            flops += block.feed_forward.flops(tokens)
     flops += 2.0 * logit_rows * model.plan.head.hidden_size * model.plan.head.vocab_size
     return flops
 
@@ -208,6 +210,40 @@ def run_stress(model, args) -> dict:
             "graph_steps": runner.graph_steps, "dtype": args.dtype}
 
 
+def run_compare(args) -> dict:
+    """Prefill and decode of pairs of shapes at equal layer sizes, one model after the other on the same
+    machine: the Tasosun shapes beside the Gemma shapes they were sized after.  Every point has its time and its
+    share of the peak (HBM for decoding, the matrix cores for prompts), as the default line's points have."""
+    import torch
+
+    from wllm_amd.cli import read_shape
+    points = {}
+    graphs = not args.no_graphs
+    for pair in args.compare.split(","):
+        for name in pair.split(":"):
+            shape = read_shape(name)
+            model = build_model(shape, args.dtype, args.seed)
+            key = os.path.basename(name).replace(".json", "")
+            points[f"{key}_weight_bytes"] = model.weight_bytes()
+            for tokens in (512, 2048, 8192):
+                mean, _ = measure_prefill(model, tokens, args.block_size, repeats=3)
+                points[f"{key}_prefill_{tokens}"] = round(tokens / mean, 1)
+                points[f"{key}_prefill_{tokens}_ms"] = round(1000.0 * mean, 3)
+                points[f"{key}_prefill_{tokens}_frac"] = round(step_flops(model, tokens, 0, 1) / mean / PEAK_FLOPS[args.dtype], 4)
+            for batch in (1, 8, 64):
+                k = max(8, args.steps // 2)
+                d, ctx_len = measure_decode(model, batch, args.context, k, 4, args.block_size, graphs)
+                gbs = (model.weight_bytes() + batch * ctx_len * kv_bytes_per_token(model)) / (d / k) / 1e9
+                points[f"{key}_decode_b{batch}"] = round(k * batch / d, 1)
+                points[f"{key}_decode_b{batch}_ms"] = round(1000.0 * d / k, 4)
+                points[f"{key}_decode_b{batch}_frac"] = round(gbs / PEAK_HBM_GBS, 4)
+            del model
+            torch.cuda.empty_cache()
+    return {"metric": "prefill and decode of pairs of shapes at equal layer sizes", "pairs": args.compare,
+            "dtype": args.dtype, "context": args.context, "hip_graphs": graphs,
+            "data": "synthetic: seeded random weights (normal, std 0.02) and seeded uniform token ids", "points": points}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -226,8 +262,11 @@ def main() -> int:
                     help="basic: batch 1 and 64 and the long context; all (default): also batch 128 and 256, batch 64 at "
                          "longer contexts, the stress workload, float32 decoding and the Gemma-7B layer sizes")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "stress"],
-                    help="decode: the contract's line; stress: continuous batching of 64 mixed requests")
+    ap.add_argument("--workload", default="decode", choices=["decode", "stress", "compare"],
+                    help="decode: the contract's line; stress: continuous batching of 64 mixed requests; compare: prefill "
+                         "and decode of the pairs of shapes of --compare, one model after the other")
+    ap.add_argument("--compare", default="tasosun-2b:gemma-2b,tasosun-7b:gemma-7b",
+                    help="compare: pairs of shapes (named, or config.json files), new:closest, with commas between pairs")
     ap.add_argument("--stress-requests", type=int, default=64)
     ap.add_argument("--row-multiple", type=int, default=256,
                     help="stress: a step's rows are trimmed to a multiple of this where the budget cuts a portion (0: off)")
@@ -247,10 +286,18 @@ def main() -> int:
     from wllm_amd.kernels import ops
 
     ops.backend()
+    if args.workload == "compare":
+        with torch.inference_mode():
+            print(json.dumps(run_compare(args)))
+        return 0
     shape = read_shape(args.shape)
-    full_layers = shape["num_hidden_layers"]
+    # a shape counts its layers (`num_hidden_layers`) or lists them (`layers`)
+    full_layers = shape["num_hidden_layers"] if "num_hidden_layers" in shape else len(shape["layers"])
     if args.layers is not None:
-        shape["num_hidden_layers"] = args.layers
+        if "num_hidden_layers" in shape:
+            shape["num_hidden_layers"] = args.layers
+        else:
+            shape["layers"] = shape["layers"][:args.layers]
     with torch.inference_mode():
         model = build_model(shape, args.dtype, args.seed)
         if args.workload == "stress":
@@ -335,7 +382,8 @@ def main() -> int:
             torch.cuda.empty_cache()
 
     c = shape
-    sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B"}.get(args.shape, os.path.basename(args.shape))
+    sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B", "tasosun-2b": "Gemma-2B (as Tasosun layers)",
+             "tasosun-7b": "Gemma-7B (as Tasosun layers)"}.get(args.shape, os.path.basename(args.shape))
     line = {
         "metric": f"decode tokens/s, {sizes} layer sizes, after {args.context:,}-token prompts",
         "value": round(value, 1),
@@ -350,7 +398,7 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic: seeded random weights (normal, std 0.02) and seeded uniform token ids",
         "config": {
-            "model": f"{sizes} layer sizes ({c['architectures'][0]}), random weights",
+            "model": f"{sizes} layer sizes ({(c.get('architectures') or [c.get('architecture')])[0]}), random weights",
             "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU",
             "layers": layers_run, "layers_of_full_model": full_layers, "hidden_size": plan.embedding.hidden_size,
             "intermediate_size": c.get("intermediate_size"), "num_attention_heads": c.get("num_attention_heads"),

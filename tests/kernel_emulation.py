@@ -182,9 +182,9 @@ class EmulatedKernels:
             v = total.to(self.acc)
         else:
             v = rows.to(self.acc)
-        if bias is not None:
-            v = v + bias.to(self.acc)
         v = v.clone()
+        if bias is not None:
+            v[:, :bias.shape[0]] += bias.to(self.acc)       # the row's first columns have a bias
         r = num_heads + num_kv_heads
         heads = v[:, :r * head_dim].reshape(n, r, head_dim).clone()
         as_projected = heads[:, num_heads:].clone()

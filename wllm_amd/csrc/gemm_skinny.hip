@@ -360,7 +360,7 @@ struct NormOnLoad {
 template <int MT, int ACT, bool TILED, int TPW, bool NORM, int XR>
 __global__ void __launch_bounds__(TPW * 128, MT == 1 ? (NORM && XR > 2 ? 3 : 4) : (MT == 2 ? 3 : 2))
 gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16* __restrict__ w, bf16* __restrict__ out,
-                         int M, int inter, int K, int chunk) {
+                         int M, int inter, int K, int chunk, int out_stride) {
     extern __shared__ uint4 xs[];                 // two halves of [MT*16][chunk/8 + 1]
     __shared__ float inv_s[16];                   // NORM: a row's rsqrt(mean square + eps)
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -534,8 +534,8 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
             const float gate = accg[t][v] + red[t * 8 + v], upv = accu[t][v] + red[t * 8 + 4 + v];
             r[v] = activate<ACT>(gate) * upv;
         }
-        bf16* o = out + static_cast<size_t>(m) * inter + n;
-        if (n + 3 < inter && (inter % 4 == 0)) {
+        bf16* o = out + static_cast<size_t>(m) * out_stride + n;     // out may be a band of columns of a wider buffer
+        if (n + 3 < inter && (inter % 4 == 0) && (out_stride % 4 == 0)) {
             store4<bf16>(o, r);
         } else {
 #pragma unroll
@@ -546,7 +546,8 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
 }
 
 static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const void* w, int tiled, void* out, int M,
-                        int inter, int K, int activation, int chunk, hipStream_t stream) {
+                        int inter, int K, int activation, int chunk, int out_stride, hipStream_t stream) {
+    if (out_stride < inter) return -1;
     if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation >= kActivations) return -1;
     const int mt = (M + 15) / 16;
     if (chunk > K / 2) chunk = K / 2;
@@ -572,7 +573,8 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
             roomy = true;                                                                                             \
         }                                                                                                             \
         gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR><<<grid, TPW * 128, smem, stream>>>(                        \
-            static_cast<const bf16*>(x), norm, static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk); \
+            static_cast<const bf16*>(x), norm, static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk, \
+            out_stride);                                                                                              \
     } while (0)
 #define LAUNCH_T(MT, A, T, TPW) LAUNCH_K(MT, A, T, TPW, false, 4)
 #define LAUNCH(MT, A)                        \
@@ -606,10 +608,13 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
     return launch_status();
 }
 
+// `out_stride`: elements between two rows of out (inter, or more where out is a band of columns of a
+// wider buffer; the band then begins at a multiple of 8 bytes).
 WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, void* out, int M, int inter, int K,
-                                    int activation, int chunk, hipStream_t stream) {
+                                    int activation, int chunk, int out_stride, hipStream_t stream) {
+    if (reinterpret_cast<uintptr_t>(out) % 8 != 0) return -1;
     return gated_launch(x, NormOnLoad{nullptr, nullptr, nullptr, 0, 0.f, 0.f}, false, w, tiled, out, M, inter, K, activation,
-                        chunk, stream);
+                        chunk, out_stride, stream);
 }
 
 // The same product with the RMS norm of the residual stream folded into the load of x: at most 16
@@ -620,5 +625,5 @@ WLLM_API int wllm_gemm_skinny_gated_norm(const float* residual, const float* sum
                                          int K, int activation, hipStream_t stream) {
     if (M > 16 || sumsq_cols < 1) return -1;
     return gated_launch(nullptr, NormOnLoad{residual, sumsq, norm_weight, sumsq_cols, eps, offset}, true, w, tiled, out, M,
-                        inter, K, activation, 256, stream);
+                        inter, K, activation, 256, inter, stream);
 }

@@ -9,36 +9,46 @@
 constexpr int kPrepareWaves = 4;
 constexpr int kPrepareMaxHead = 256;
 constexpr int kPerLane = kPrepareMaxHead / kWave;
+constexpr int kRestColumns = kWave * kPrepareWaves * 4;      // columns beyond the heads that one workgroup takes
 
-// One workgroup per token, one wavefront per head at a time.  A row is
-//   [num_heads query heads | num_kv_heads key heads | num_kv_heads value heads, unless the values are the keys | extra]
+template <typename T> struct alignas(4 * sizeof(T)) Four { T v[4]; };
+
+// A row is
+//   [num_heads query heads | num_kv_heads key heads | num_kv_heads value heads, unless the values are the keys | the rest]
 // of head_dim elements a head.  In the order of the steps, for every query and key head:
-//   1. the element is the row's (or the sum of the stack of partial sums `parts`), plus its bias;
+//   1. the element is the row's (or the sum of the stack of partial sums `parts`), plus its bias
+//      (the bias covers the row's first bias_width columns);
 //   2. where the values are the keys, the key head as it is now goes to the cache's values;
 //   3. the first rotary_dim elements turn by position * inv_freq[j]: pair j is (2j, 2j + 1)
 //      (interleaved) or (j, j + rotary_dim / 2);
 //   4. with norm_eps >= 0 the head is divided by sqrt(mean of its squares + norm_eps);
 //   5. it is written back to the row, and a key head to the cache's keys.
-// Value heads of their own and the extra columns take step 1 only.  Keys lie in the cache as
+// Value heads of their own and the rest of the row take step 1 only.  Keys lie in the cache as
 // [page_size, head_dim], values transposed as [head_dim, page_size].
-template <typename T>
+//
+// The grid is (token, piece): the first pieces are groups of four heads, a wavefront a head; the others
+// take kRestColumns columns each of what lies behind the query and key heads.  A decode step's few
+// tokens so fill some tens of workgroups instead of one a token, whose wavefronts would walk the heads
+// and the stack of partial sums one after the other.  FOUR: head_dim and the row's width are multiples
+// of four and the pairs are neighbours (or nothing turns), so a lane owns four consecutive elements with
+// both partners of its pairs and moves 8 or 16 bytes at a time; else a lane owns elements 64 apart and
+// finds a partner in shared memory.
+template <typename T, bool FOUR>
 __global__ void __launch_bounds__(kWave * kPrepareWaves)
 head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict__ parts, int splits, size_t split_stride,
-                    const float* __restrict__ bias, const int* __restrict__ positions,
+                    const float* __restrict__ bias, int bias_width, const int* __restrict__ positions,
                     const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ cache,
                     long long num_pages, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
-                    int interleaved, float norm_eps, int values_are_keys, int page_size) {
-    __shared__ float staged[kPrepareWaves][kPrepareMaxHead];
+                    int interleaved, float norm_eps, int values_are_keys, int page_size, int head_pieces) {
+    __shared__ float staged[kPrepareWaves][FOUR ? 1 : kPrepareMaxHead];
     const int token = blockIdx.x;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     T* row = rows + static_cast<size_t>(token) * row_width;
     const float* prow = parts ? parts + static_cast<size_t>(token) * row_width : nullptr;
     auto value = [&](int idx) -> float {
         const float v = prow ? stack_sum(prow + idx, splits, split_stride) : to_float(row[idx]);
-        return bias ? v + bias[idx] : v;
+        return idx < bias_width ? v + bias[idx] : v;
     };
-    const bool rewrite = bias || prow;
-    const float pos = static_cast<float>(positions[token]);
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * head_dim;
     T* kpage = nullptr;
     T* vpage = nullptr;
@@ -52,104 +62,177 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
             vpage = kpage + static_cast<size_t>(num_kv_heads) * page_size * head_dim;
         }
     }
-    // the lane's elements of a head are lane, lane + 64, ...; their angles do not depend on the head
+    const int turned_heads = num_heads + num_kv_heads;
+    if (static_cast<int>(blockIdx.y) >= head_pieces) {
+        // ---- behind the query and key heads: value heads of their own, then the rest of the row ----
+        const int begin = turned_heads * head_dim;
+        const int values_end = values_are_keys ? begin : begin + num_kv_heads * head_dim;
+        const int idx0 = begin + (static_cast<int>(blockIdx.y) - head_pieces) * kRestColumns + threadIdx.x * 4;
+        for (int u = 0; u < 4; ++u) {
+            const int idx = idx0 + u;
+            if (idx >= row_width) break;
+            const bool rewrite = prow || idx < bias_width;
+            if (!rewrite && !(idx < values_end && vpage)) continue;
+            T v = row[idx];
+            if (rewrite) {
+                v = from_float<T>(value(idx));
+                row[idx] = v;
+            }
+            if (idx < values_end && vpage) {
+                const int head = (idx - begin) / head_dim, j = (idx - begin) % head_dim;
+                vpage[(static_cast<size_t>(head) * head_dim + j) * page_size + off] = v;
+            }
+        }
+        return;
+    }
+    const int head = static_cast<int>(blockIdx.y) * kPrepareWaves + wave;
+    if (head >= turned_heads) return;
+    const float pos = static_cast<float>(positions[token]);
+    const int base = head * head_dim;
+    const int kvh = head - num_heads;                 // >= 0: a key head
     const int half = rotary_dim / 2;
-    float sn[kPerLane], cs[kPerLane];
+    if (FOUR) {
+        const int e = 4 * lane;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        const bool live = e < head_dim;
+        if (live) {
+            if (prow) {
+                // the partial sums are added in stack order, eight slices asked for at a time
+                const float* p = prow + base + e;
+                Four<float> t = *reinterpret_cast<const Four<float>*>(p);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = t.v[u];
+                for (int s0 = 1; s0 < splits; s0 += 8) {
+                    Four<float> q[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        q[j] = *reinterpret_cast<const Four<float>*>(p + static_cast<size_t>(min(s0 + j, splits - 1)) * split_stride);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (s0 + j >= splits) break;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] += q[j].v[u];
+                    }
+                }
+            } else {
+                const Four<T> t = *reinterpret_cast<const Four<T>*>(row + base + e);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = to_float(t.v[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (base + e + u < bias_width) v[u] += bias[base + e + u];
+            if (values_are_keys && kvh >= 0 && vpage) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    vpage[(static_cast<size_t>(kvh) * head_dim + e + u) * page_size + off] = from_float<T>(v[u]);
+            }
+            if (inv_freq) {
+#pragma unroll
+                for (int u = 0; u < 4; u += 2) {
+                    if (e + u < rotary_dim) {
+                        float sn, cs, ra, rb;
+                        sincosf(pos * inv_freq[(e + u) >> 1], &sn, &cs);
+                        rotate_pair(v[u], v[u + 1], sn, cs, ra, rb);
+                        v[u] = ra;
+                        v[u + 1] = rb;
+                    }
+                }
+            }
+        }
+        float inv = 1.f;
+        if (norm_eps >= 0.f) {
+            const float ss = wave_sum(v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3]);
+            inv = rsqrtf(ss / static_cast<float>(head_dim) + norm_eps);
+        }
+        if (live) {
+            Four<T> r;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) r.v[u] = from_float<T>(v[u] * inv);
+            *reinterpret_cast<Four<T>*>(row + base + e) = r;
+            if (kvh >= 0 && kpage)
+                *reinterpret_cast<Four<T>*>(kpage + (static_cast<size_t>(kvh) * page_size + off) * head_dim + e) = r;
+        }
+        return;
+    }
+    // ---- any sizes, either pairing: the lane's elements are lane, lane + 64, ... ----
+    float* mine = staged[wave];
+    float v[kPerLane];
 #pragma unroll
     for (int k = 0; k < kPerLane; ++k) {
         const int e = lane + k * kWave;
-        sn[k] = 0.f;
-        cs[k] = 1.f;
+        v[k] = e < head_dim ? value(base + e) : 0.f;
+        if (e < head_dim) mine[e] = v[k];
+        if (values_are_keys && kvh >= 0 && vpage && e < head_dim)
+            vpage[(static_cast<size_t>(kvh) * head_dim + e) * page_size + off] = from_float<T>(v[k]);
+    }
+    // lanes read below what other lanes of the wavefront wrote above
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+        const int e = lane + k * kWave;
         if (inv_freq && e < rotary_dim) {
-            const int j = interleaved ? e >> 1 : (e < half ? e : e - half);
-            sincosf(pos * inv_freq[j], &sn[k], &cs[k]);
+            const bool first = interleaved ? (e & 1) == 0 : e < half;
+            const int partner = interleaved ? (e ^ 1) : (first ? e + half : e - half);
+            const int j = interleaved ? e >> 1 : (first ? e : e - half);
+            const float other = mine[partner];
+            float sn, cs, ra, rb;
+            sincosf(pos * inv_freq[j], &sn, &cs);
+            rotate_pair(first ? v[k] : other, first ? other : v[k], sn, cs, ra, rb);
+            v[k] = first ? ra : rb;
+        }
+        ss += v[k] * v[k];
+    }
+    float inv = 1.f;
+    if (norm_eps >= 0.f) inv = rsqrtf(wave_sum(ss) / static_cast<float>(head_dim) + norm_eps);
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+        const int e = lane + k * kWave;
+        if (e < head_dim) {
+            const T r = from_float<T>(v[k] * inv);
+            row[base + e] = r;
+            if (kvh >= 0 && kpage) kpage[(static_cast<size_t>(kvh) * page_size + off) * head_dim + e] = r;
         }
     }
-    float* mine = staged[wave];
-    const int turned_heads = num_heads + num_kv_heads;
-    for (int head = wave; head < turned_heads; head += kPrepareWaves) {
-        const int base = head * head_dim;
-        const int kvh = head - num_heads;                 // >= 0: a key head
-        float v[kPerLane];
-#pragma unroll
-        for (int k = 0; k < kPerLane; ++k) {
-            const int e = lane + k * kWave;
-            v[k] = e < head_dim ? value(base + e) : 0.f;
-            if (e < head_dim) mine[e] = v[k];
-            if (values_are_keys && kvh >= 0 && vpage && e < head_dim)
-                vpage[(static_cast<size_t>(kvh) * head_dim + e) * page_size + off] = from_float<T>(v[k]);
-        }
-        // lanes read below what other lanes of the wavefront wrote above
-        __builtin_amdgcn_wave_barrier();
-        asm volatile("" ::: "memory");
-        float ss = 0.f;
-#pragma unroll
-        for (int k = 0; k < kPerLane; ++k) {
-            const int e = lane + k * kWave;
-            if (inv_freq && e < rotary_dim) {
-                const bool first = interleaved ? (e & 1) == 0 : e < half;
-                const int partner = interleaved ? (e ^ 1) : (first ? e + half : e - half);
-                const float other = mine[partner];
-                float ra, rb;
-                rotate_pair(first ? v[k] : other, first ? other : v[k], sn[k], cs[k], ra, rb);
-                v[k] = first ? ra : rb;
-            }
-            ss += v[k] * v[k];
-        }
-        float inv = 1.f;
-        if (norm_eps >= 0.f) inv = rsqrtf(wave_sum(ss) / static_cast<float>(head_dim) + norm_eps);
-#pragma unroll
-        for (int k = 0; k < kPerLane; ++k) {
-            const int e = lane + k * kWave;
-            if (e < head_dim) {
-                const T r = from_float<T>(v[k] * inv);
-                row[base + e] = r;
-                if (kvh >= 0 && kpage) kpage[(static_cast<size_t>(kvh) * page_size + off) * head_dim + e] = r;
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        asm volatile("" ::: "memory");
-    }
-    // value heads of their own
-    int done = turned_heads * head_dim;
-    if (!values_are_keys) {
-        if (rewrite || vpage) {
-            for (int idx = threadIdx.x; idx < num_kv_heads * head_dim; idx += blockDim.x) {
-                const int head = idx / head_dim, j = idx % head_dim;
-                T v = row[done + idx];
-                if (rewrite) {
-                    v = from_float<T>(value(done + idx));
-                    row[done + idx] = v;
-                }
-                if (vpage) vpage[(static_cast<size_t>(head) * head_dim + j) * page_size + off] = v;
-            }
-        }
-        done += num_kv_heads * head_dim;
-    }
-    // what lies beyond the heads
-    if (rewrite)
-        for (int idx = done + threadIdx.x; idx < row_width; idx += blockDim.x) row[idx] = from_float<T>(value(idx));
 }
 
-// Returns 0, a HIP error code, or -1 for sizes the kernel does not take.
+// Returns 0, a HIP error code, or -1 for sizes the kernel does not take.  `bias` covers the first
+// `bias_width` columns of a row (0: no bias).
 WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const float* parts, int splits,
-                               long long split_stride, const float* bias, const int* positions, const float* inv_freq,
-                               const int* slots, void* cache, long long num_pages, int n, int num_heads,
-                               int num_kv_heads, int head_dim, int rotary_dim, int interleaved, float norm_eps,
-                               int values_are_keys, int page_size, hipStream_t stream) {
+                               long long split_stride, const float* bias, int bias_width, const int* positions,
+                               const float* inv_freq, const int* slots, void* cache, long long num_pages, int n,
+                               int num_heads, int num_kv_heads, int head_dim, int rotary_dim, int interleaved,
+                               float norm_eps, int values_are_keys, int page_size, hipStream_t stream) {
     const int heads = num_heads + (values_are_keys ? 1 : 2) * num_kv_heads;
     if (head_dim <= 0 || head_dim > kPrepareMaxHead || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 != 0 ||
-        row_width < heads * head_dim || num_heads < 0 || num_kv_heads < 0 || page_size <= 0)
+        row_width < heads * head_dim || num_heads < 0 || num_kv_heads < 0 || page_size <= 0 || bias_width < 0 ||
+        bias_width > row_width || (bias == nullptr && bias_width != 0))
         return -1;
     if (inv_freq == nullptr && rotary_dim != 0) return -1;
     if (n <= 0) return 0;
-#define LAUNCH(T)                                                                                                   \
-    head_prepare_kernel<T><<<n, kWave * kPrepareWaves, 0, stream>>>(                                                \
-        static_cast<T*>(rows), row_width, parts, splits, static_cast<size_t>(split_stride), bias, positions, inv_freq, \
-        slots, static_cast<T*>(cache), num_pages, num_heads, num_kv_heads, head_dim, rotary_dim, interleaved, norm_eps, \
-        values_are_keys, page_size)
-    if (is_bf16) LAUNCH(bf16);
-    else LAUNCH(float);
+    const int turned = (num_heads + num_kv_heads) * head_dim;
+    const int head_pieces = (num_heads + num_kv_heads + kPrepareWaves - 1) / kPrepareWaves;
+    // what lies behind the query and key heads needs a workgroup only if something is to be done there
+    const bool rest = row_width > turned && (parts != nullptr || bias_width > turned || (!values_are_keys && cache != nullptr));
+    const int rest_pieces = rest ? (row_width - turned + kRestColumns - 1) / kRestColumns : 0;
+    if (head_pieces + rest_pieces > 65535) return -1;
+    const dim3 grid(n, head_pieces + rest_pieces);
+    const bool four = head_dim % 4 == 0 && row_width % 4 == 0 && (interleaved || rotary_dim == 0) &&
+                      (parts == nullptr || split_stride % 4 == 0) &&
+                      reinterpret_cast<uintptr_t>(rows) % 16 == 0 && reinterpret_cast<uintptr_t>(parts) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(cache) % 16 == 0;
+#define LAUNCH(T, FOUR)                                                                                             \
+    head_prepare_kernel<T, FOUR><<<grid, kWave * kPrepareWaves, 0, stream>>>(                                       \
+        static_cast<T*>(rows), row_width, parts, splits, static_cast<size_t>(split_stride), bias, bias_width, positions, \
+        inv_freq, slots, static_cast<T*>(cache), num_pages, num_heads, num_kv_heads, head_dim, rotary_dim, interleaved, \
+        norm_eps, values_are_keys, page_size, head_pieces)
+    if (is_bf16) {
+        if (four) LAUNCH(bf16, true); else LAUNCH(bf16, false);
+    } else {
+        if (four) LAUNCH(float, true); else LAUNCH(float, false);
+    }
 #undef LAUNCH
     return launch_status();
 }

@@ -36,7 +36,7 @@ _SIGNATURES = {
                       c_int, c_float, c_float, c_void_p],
     "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_gemm_skinny_gated_norm": [c_void_p, c_void_p, c_int, c_void_p, c_float, c_float, c_void_p, c_int, c_void_p, c_int,
                                     c_int, c_int, c_int, c_void_p],
     "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -464,10 +464,10 @@ class HipBackend:
             _ptr(partial), m, n, x.shape[1], self._stream()), "linear")
 
     def gated_linear_writes_band(self, rows: int, dtype, in_features: int) -> bool:
-        """True where `gated_linear` runs the product and the activation as two kernels: the second
-        writes rows of any stride."""
+        """True where `gated_linear` runs a kernel that writes rows of any stride: the few-row product, and
+        the activation kernel where the product and the activation are two kernels."""
         if self.skinny_takes(dtype, rows, in_features) and in_features % 64 == 0:
-            return False
+            return True        # the few-row kernel takes a row stride for its result
         return not (dtype == torch.bfloat16 and 64 < rows <= self.TILE_GATED_MAX_ROWS and in_features % 64 == 0)
 
     def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
@@ -477,7 +477,8 @@ class HipBackend:
         if self.skinny_takes(x.dtype, m, k) and k % 64 == 0:
             self._check(self.lib.wllm_gemm_skinny_gated(
                 _ptr(x), _ptr(w), tiled, _ptr(out), m, out.shape[1], k, ACTIVATIONS[activation],
-                self.GATED_CHUNK[-(-m // 16)], self._stream()), "gated_linear (few rows, matrix cores)")
+                self.GATED_CHUNK[-(-m // 16)], out.stride(0) if m > 1 else out.shape[1], self._stream()),
+                "gated_linear (few rows, matrix cores)")
             return
         n = out.shape[1]
         if (x.dtype == torch.bfloat16 and 64 < m <= self.TILE_GATED_MAX_ROWS and k % 64 == 0

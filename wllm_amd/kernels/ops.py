@@ -350,7 +350,8 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
     """What `rope_and_cache_write` does, for attention blocks that do more between projection and
     attention.  rows T [n, width]: num_heads query heads, num_kv_heads key heads, num_kv_heads value
     heads unless `values_are_keys`, then any further columns.  In this order, in float32: every
-    element takes its bias (float32 [width] or None) and, with `parts` (float32 [S, n, width]), is
+    element takes its bias (float32 [w] with w <= width: the row's first w columns have one; or None)
+    and, with `parts` (float32 [S, n, width]), is
     the sum of the stack in order instead of what the row held; with `values_are_keys` a key head
     as it is now is stored as the value head; the first 2 * len(inv_freq) elements of every query
     and key head turn by position * inv_freq[j], pair j being elements (2j, 2j + 1) if
@@ -364,7 +365,8 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
     n, width = rows.shape
     _need(0 < head_dim <= 256, "head_dim: at most 256")
     if bias is not None:
-        _dense(bias, "bias", torch.float32, (width,))
+        _dense(bias, "bias", torch.float32)
+        _need(bias.dim() == 1 and 0 < bias.shape[0] <= width, lambda: f"bias: shape {tuple(bias.shape)}, expected at most [{width}]")
     if parts is not None:
         _need(parts.dim() == 3 and parts.shape[0] >= 1, "parts: expected [S, n, width]")
         _dense(parts, "parts", torch.float32, (parts.shape[0], n, width))
@@ -583,8 +585,8 @@ def gated_linear_norm_takes(rows: int, dtype: torch.dtype, in_features: int) -> 
 
 
 def gated_linear_writes_band(rows: int, dtype: torch.dtype, in_features: int) -> bool:
-    """Whether `gated_linear` at these sizes can write `out` as a band of columns of a wider tensor (it
-    can where the product and the activation are two kernels)."""
+    """Whether `gated_linear` at these sizes can write `out` as a band of columns of a wider tensor whose
+    rows begin at multiples of 16 bytes."""
     return bool(getattr(backend(), "gated_linear_writes_band", lambda *a: False)(rows, dtype, in_features))
 
 
@@ -687,13 +689,13 @@ def _register_own() -> None:
                 page_size, interleaved, norm_eps, values_are_keys, parts):
         splits, stride = (parts.shape[0], parts.shape[1] * parts.shape[2]) if parts is not None else (0, 0)
         return fn(p(rows), int(rows.dtype == torch.bfloat16), rows.shape[1], p(parts), splits, stride, p(bias),
-                  p(positions), p(inv_freq), p(slots), p(cache), cache.shape[0] if cache is not None else 0,
+                  bias.shape[0] if bias is not None else 0, p(positions), p(inv_freq), p(slots), p(cache), cache.shape[0] if cache is not None else 0,
                   rows.shape[0], num_heads, num_kv_heads, head_dim,
                   2 * inv_freq.shape[0] if inv_freq is not None else 0, int(interleaved),
                   float(norm_eps) if norm_eps is not None else -1.0, int(values_are_keys), page_size, stream)
 
     register_op("head_prepare", entry_point="wllm_head_prepare",
-                argtypes=[c_void_p, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
+                argtypes=[c_void_p, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
                 launch=prepare)
     register_op("sigmoid_gate", entry_point="wllm_sigmoid_gate",

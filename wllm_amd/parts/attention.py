@@ -100,9 +100,10 @@ class PagedAttention:
         if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
             q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
             biases = [(s.q_bias, q), (s.k_bias, kv)] + ([] if s.values_are_keys else [(s.v_bias, kv)])
-            parts = [fetch.vector(name) if name is not None else torch.zeros(width) for name, width in biases]
-            if s.gate_weight:
-                parts.append(torch.zeros(q))
+            # (the gate's projection, behind the heads in the row, has none: the bias is shorter than the row)
+            found = [fetch.vector(name) if name is not None else None for name, _ in biases]
+            where = next(v.device for v in found if v is not None)      # a fetcher may make its tensors on the device
+            parts = [v if v is not None else torch.zeros(width, device=where) for v, (_, width) in zip(found, biases)]
             self.b_qkv = fetch.to_device(torch.cat(parts))
         if hasattr(self.position, "load"):
             self.position.load(fetch)

@@ -55,8 +55,9 @@ class GatedMLP:
             ops.gated_linear(h, self.w_gate_up, act, s.activation, None, self.t_gate_up)
         else:
             gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
-            if product_input is not None and ops.gated_linear_writes_band(n, h.dtype, s.hidden_size):
-                act = product_input         # the activation kernel writes the band itself
+            if (product_input is not None and ops.gated_linear_writes_band(n, h.dtype, s.hidden_size)
+                    and product_input.data_ptr() % 16 == 0 and product_input.stride(0) % 8 == 0):
+                act = product_input         # the kernel writes the band itself (its rows begin at multiples of 16 bytes)
             else:
                 act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
             ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up, self.t_gate_up)
