@@ -134,7 +134,7 @@ class EmulatedKernels:
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
-                        plan=None, softcap=0.0):
+                        plan=None, softcap=0.0, exact_weights=False):
         self._count("paged_attention")
         n = qkv.shape[0]
         n_rep = num_heads // num_kv_heads

@@ -138,7 +138,7 @@ def test_capped_scores_in_every_attention_kernel(dtype, nh, nkv, d, ps, window, 
     out = torch.zeros(rows.shape[0], nh * d, dtype=dtype, device=DEV)
     args = [t.to(DEV) for t in (rows, cache, bt, tok_seg, q_start, q_len, ctx)] + [out]
     kwargs = dict(num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps, scale=scale, window=window, softcap=cap,
-                  max_q_len=int(q_len.max()), max_ctx_len=int(ctx.max()))
+                  max_q_len=int(q_len.max()), max_ctx_len=int(ctx.max()), exact_weights=True)
     kwargs["plan"] = ops.plan_paged_attention(q_len.numpy(), ctx.numpy(), num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps,
                                               window=window, dtype=dtype, device=torch.device(DEV))
     ops.paged_attention(*args, **kwargs)
@@ -163,6 +163,42 @@ def test_capped_scores_in_every_attention_kernel(dtype, nh, nkv, d, ps, window, 
             close(out[int(q_start[s]):int(q_start[s]) + ql, head * d:(head + 1) * d], p @ values[:, kv], dtype,
                   f"segment {s} head {head}")
     assert bent > 0, "no score came near the cap: the case would pass without it"
+
+
+@pytest.mark.parametrize("segs", [[(1, 3)] * 150, [(70, 70), (64, 67)]])
+def test_bfloat16_kernels_weigh_the_values_with_more_than_bfloat16(segs):
+    """With `exact_weights` the matrix-core kernels' only rounding is that of their result: their distance from
+    the exact weighted sum is that of the exact sum's own rounding to bfloat16.  Without it the rounding of
+    the weights shows on top (so the case can tell the two apart)."""
+    nh, nkv, d, ps = 4, 2, 64, 16
+    rows, cache, bt, tok_seg, q_start, q_len, ctx = _attention_problem(torch.bfloat16, nh, nkv, d, ps, segs, seed=9, extra_columns=0)
+    window = 3          # few keys a query: single weights count
+    dev = [t.to(DEV) for t in (rows, cache, bt, tok_seg, q_start, q_len, ctx)]
+    plan = ops.plan_paged_attention(q_len.numpy(), ctx.numpy(), num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps,
+                                    window=window, dtype=torch.bfloat16, device=torch.device(DEV))
+    got = {}
+    for exact in (True, False):
+        out = torch.zeros(rows.shape[0], nh * d, dtype=torch.bfloat16, device=DEV)
+        ops.paged_attention(*dev, out, num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps, scale=0.2, window=window,
+                            max_q_len=int(q_len.max()), max_ctx_len=int(ctx.max()), plan=plan, exact_weights=exact)
+        got[exact] = out.double().cpu()
+    want = torch.zeros(rows.shape[0], nh * d, dtype=torch.float64)
+    kview, vview = cache[:, 0].view(-1, nkv, ps, d).double(), cache[:, 1].view(-1, nkv, d, ps).double()
+    for s, (ql, cl) in enumerate(segs):
+        ids = bt[s, :-(-cl // ps)].long()
+        keys = kview[ids].permute(0, 2, 1, 3).reshape(-1, nkv, d)[:cl]
+        values = vview[ids].permute(0, 3, 1, 2).reshape(-1, nkv, d)[:cl]
+        mask = tasosun_plain.window_mask(torch.arange(cl), window)[cl - ql:]
+        q = rows[int(q_start[s]):int(q_start[s]) + ql].double().view(ql, nh, d)
+        for head in range(nh):
+            kv = head // (nh // nkv)
+            sc = (q[:, head] @ keys[:, kv].T * 0.2).masked_fill(~mask, float("-inf"))
+            want[int(q_start[s]):int(q_start[s]) + ql, head * d:(head + 1) * d] = torch.softmax(sc, -1) @ values[:, kv]
+    rounding = (want.to(torch.bfloat16).double() - want).pow(2).mean().sqrt().item()
+    exact_err = (got[True] - want).pow(2).mean().sqrt().item()
+    rounded_err = (got[False] - want).pow(2).mean().sqrt().item()
+    assert exact_err <= 1.01 * rounding, (exact_err, rounding)
+    assert rounded_err > 1.04 * rounding, (rounded_err, rounding)     # (measured: 1.05 to 1.06)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

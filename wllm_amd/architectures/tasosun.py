@@ -50,7 +50,7 @@ def tasosun_plan(cfg: TasosunConfig) -> ModelPlan:
                 window=a.window, position=position,
                 q_weight=p + "mix.q", k_weight=p + "mix.k", o_weight=p + "mix.o", gate_weight=p + "mix.g",
                 q_bias=p + "mix.q.b", k_bias=p + "mix.k.b", o_bias=p + "mix.o.b",
-                softcap=a.softcap, qk_norm_eps=cfg.norm_eps, values_are_keys=True),
+                softcap=a.softcap, qk_norm_eps=cfg.norm_eps, values_are_keys=True, weights_in_float32=True),
             feed_forward=None if layer.ff is None else GatedMLPSpec(
                 hidden_size=cfg.width, intermediate_size=layer.ff, activation="silu",
                 gate_weight=p + "mlp.gate", up_weight=p + "mlp.up", down_weight=p + "mlp.down"),

@@ -56,7 +56,8 @@ __device__ __forceinline__ uint16_t bf16_bits(float f) { return from_float<bf16>
 
 // Three workgroups a compute unit (168 registers a lane) where the kernel fits them without spilling;
 // two for the head sizes and page sizes whose staging needs more.
-template <int HD, bool V16>
+// SPLIT: the weights of the second product keep 16 bits (rounded weight and remainder, two products).
+template <int HD, bool V16, bool SPLIT>
 __global__ void __launch_bounds__(256, (HD <= 160 || (HD == 256 && V16)) ? 3 : 2)
 paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                             const int* __restrict__ block_tables, const int* __restrict__ items,
@@ -220,7 +221,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             const int key = kbase + (V16 ? 8 * g + 4 * t2 + v : 16 * t2 + 4 * g + v);
             ok[e] = row_valid && key <= pos && key >= lo && key >= key_begin && key < key_end;
             // with a cap the score is scaled and bent here, and `scale_log2e` is log2(e) alone
-            sv[e] = softcap > 0.f ? softcap * tanhf(s[t2][v] * cap_scale) : s[t2][v];
+            sv[e] = softcap > 0.f ? capped_score_fast(s[t2][v] * cap_scale, softcap) : s[t2][v];
             if (ok[e]) tile_max = fmaxf(tile_max, sv[e]);
         }
         tile_max = max_across(max_across(tile_max, 16), 32);
@@ -235,6 +236,12 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         }
         pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
                           pack2_bf16(pe[6], pe[7]));
+        Pack16 pr;      // SPLIT: what the rounding left out
+        if (SPLIT)
+            pr.u = make_uint4(pack2_bf16(bf16_remainder(pe[0]), bf16_remainder(pe[1])),
+                              pack2_bf16(bf16_remainder(pe[2]), bf16_remainder(pe[3])),
+                              pack2_bf16(bf16_remainder(pe[4]), bf16_remainder(pe[5])),
+                              pack2_bf16(bf16_remainder(pe[6]), bf16_remainder(pe[7])));
         // the row's sum over its four lanes
         l_run = sum_across(sum_across(l_run, 16), 32);
         // ---- out^T = V^T . P^T ----
@@ -251,6 +258,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                 }
             }
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            if (SPLIT) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pr.v, acc[t], 0, 0, 0);
         }
     } else {
 #pragma unroll
@@ -464,12 +472,13 @@ struct AttentionArguments {
     int window;
     int q_stride;
     float cap_scale, softcap;
+    int split_weights;
     hipStream_t stream;
 };
 
-template <int HD, bool V16>
+template <int HD, bool V16, bool SPLIT>
 int launch_items(const AttentionArguments& a) {
-    paged_attention_mfma_kernel<HD, V16><<<a.num_items, 256, 0, a.stream>>>(
+    paged_attention_mfma_kernel<HD, V16, SPLIT><<<a.num_items, 256, 0, a.stream>>>(
         a.qkv, a.cache, a.block_tables, a.items, a.live_items, a.seg_q_start, a.seg_q_len, a.seg_ctx_len, a.out,
         a.partial_o, a.partial_ml, a.num_heads, a.num_kv_heads, a.page_size, a.max_pages, a.scale_log2e, a.window,
         a.q_stride, a.cap_scale, a.softcap);
@@ -479,7 +488,9 @@ int launch_items(const AttentionArguments& a) {
 template <int HD>
 int launch_all(const AttentionArguments& a) {
     if (a.num_items > 0) {
-        const int status = a.page_size % 8 == 0 ? launch_items<HD, true>(a) : launch_items<HD, false>(a);
+        const int status = a.page_size % 8 == 0
+            ? (a.split_weights ? launch_items<HD, true, true>(a) : launch_items<HD, true, false>(a))
+            : (a.split_weights ? launch_items<HD, false, true>(a) : launch_items<HD, false, false>(a));
         if (status != 0) return status;
     }
     if (a.num_reduce_items >= 64) {
@@ -503,7 +514,8 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
                                        int num_reduce_items, const int* seg_q_start, const int* seg_q_len,
                                        const int* seg_ctx_len, void* out, float* partial_o, float* partial_ml,
                                        int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
-                                       float scale, int window, int q_stride, float softcap, hipStream_t stream) {
+                                       float scale, int window, int q_stride, float softcap, int split_weights,
+                                       hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         num_heads >= (1 << 16))       // an item holds a key/value head and a tile's first row in 16 bits each
         return -1;
@@ -515,7 +527,7 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
                                   live_items, num_items, reduce_items, num_reduce_items, seg_q_start, seg_q_len,
                                   seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads,
                                   page_size, max_pages, in_exponent * 1.4426950408889634f, window, q_stride, cap_scale,
-                                  softcap, stream};
+                                  softcap, split_weights, stream};
     switch (head_dim) {
         case 32: return launch_all<32>(a);
         case 64: return launch_all<64>(a);

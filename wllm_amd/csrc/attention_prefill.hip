@@ -43,7 +43,9 @@ struct PrefillSmem {
 // the keys of its rows and writes the result itself), 2 unused.  Items that split the keys of a
 // block of rows write, per tile of 16 rows, an unnormalised accumulator and (maximum, sum) into
 // slot `partial slot + tile`, which `attention_reduce_kernel` combines.
-template <int HD, int RTW>      // RTW: tiles of 16 rows per wavefront (1 or 2)
+// RTW: tiles of 16 rows per wavefront (1 or 2).  SPLIT: the weights of the second product keep 16 bits (the
+// rounded weight and what the rounding left out, two products).
+template <int HD, int RTW, bool SPLIT>
 __global__ void __launch_bounds__(kPrefillThreads, RTW == 1 ? 2 : 1)
 paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                                const int* __restrict__ block_tables, const int* __restrict__ items,
@@ -238,7 +240,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             for (int rt = 0; rt < RTW; ++rt) s[rt][t2] = sc[rt];
         }
         // ---- softmax bookkeeping per row tile ----
-        PPack pv[RTW];
+        PPack pv[RTW], pr[RTW];
         float alpha[RTW];
         bool rescale[RTW];
 #pragma unroll
@@ -248,7 +250,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             for (int e = 0; e < 8; ++e) sv[e] = s[rt][e / 4][e % 4];
             if (softcap > 0.f) {        // the score is scaled and bent here; `scale_log2e` is then log2(e) alone
 #pragma unroll
-                for (int e = 0; e < 8; ++e) sv[e] = softcap * tanhf(sv[e] * cap_scale);
+                for (int e = 0; e < 8; ++e) sv[e] = capped_score_fast(sv[e] * cap_scale, softcap);
             }
             // blocks that lie wholly inside every row's range need no mask (a wavefront-wide decision)
             const bool inside = kbase + kBlockKeys - 1 <= t_pos_min[rt] && kbase >= t_lo_max[rt];
@@ -274,6 +276,11 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             }
             pv[rt].u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
                                   pack2_bf16(pe[6], pe[7]));
+            if (SPLIT)
+                pr[rt].u = make_uint4(pack2_bf16(bf16_remainder(pe[0]), bf16_remainder(pe[1])),
+                                      pack2_bf16(bf16_remainder(pe[2]), bf16_remainder(pe[3])),
+                                      pack2_bf16(bf16_remainder(pe[4]), bf16_remainder(pe[5])),
+                                      pack2_bf16(bf16_remainder(pe[6]), bf16_remainder(pe[7])));
             l_run[rt] = l_run[rt] * alpha[rt] + psum;
             m_run[rt] = m_new;
             rescale[rt] = __any(alpha[rt] != 1.f);
@@ -292,7 +299,10 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             a.u = *reinterpret_cast<const uint4*>(&v_s[(16 * t + i) * SV + 8 * g]);
 #pragma unroll
             for (int rt = 0; rt < RTW; ++rt)
+            {
                 acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv[rt].v, acc[rt][t], 0, 0, 0);
+                if (SPLIT) acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pr[rt].v, acc[rt][t], 0, 0, 0);
+            }
         }
     }
 #pragma unroll
@@ -371,7 +381,7 @@ __device__ __forceinline__ uint32_t shared_address(const void* p) {
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p)));
 }
 
-template <int HD>
+template <int HD, bool SPLIT>
 __global__ void __launch_bounds__(kPrefillThreads, 2)
 paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                                    const int* __restrict__ block_tables, const int* __restrict__ items,
@@ -563,7 +573,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
         }
         if (softcap > 0.f) {            // the score is scaled and bent here; `scale_log2e` is then log2(e) alone
 #pragma unroll
-            for (int e = 0; e < 8; ++e) sv[e] = softcap * tanhf(sv[e] * cap_scale);
+            for (int e = 0; e < 8; ++e) sv[e] = capped_score_fast(sv[e] * cap_scale, softcap);
         }
 #pragma unroll
         for (int t = 0; t < DT; ++t) vf[t].u = *reinterpret_cast<const uint4*>(&v_s[v_lane + 16 * t * 4 * 8]);
@@ -591,6 +601,12 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
         }
         PPack pv;
         pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]), pack2_bf16(pe[6], pe[7]));
+        PPack pr;       // SPLIT: what the rounding left out
+        if (SPLIT)
+            pr.u = make_uint4(pack2_bf16(bf16_remainder(pe[0]), bf16_remainder(pe[1])),
+                              pack2_bf16(bf16_remainder(pe[2]), bf16_remainder(pe[3])),
+                              pack2_bf16(bf16_remainder(pe[4]), bf16_remainder(pe[5])),
+                              pack2_bf16(bf16_remainder(pe[6]), bf16_remainder(pe[7])));
         l_run = l_run * alpha + psum;
         m_run = m_new;
         // ---- out^T += V^T . P^T; the accumulators are rescaled only when some row's maximum moved: one
@@ -602,7 +618,10 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < DT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pv.v, acc[t], 0, 0, 0);
+        for (int t = 0; t < DT; ++t) {
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pv.v, acc[t], 0, 0, 0);
+            if (SPLIT) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pr.v, acc[t], 0, 0, 0);
+        }
     };
     for (int blk = blk_first; blk < blk_end; blk += 2) {
         block(blk, k_s0, v_s0, 1);
@@ -637,7 +656,8 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
                                           const int* seg_q_len, const int* seg_ctx_len, void* out, float* partial_o,
                                           float* partial_ml, int num_heads,
                                           int num_kv_heads, int head_dim, int page_size, int max_pages, float scale,
-                                          int window, int q_stride, float softcap, hipStream_t stream) {
+                                          int window, int q_stride, float softcap, int split_weights,
+                                          hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
         return -1;
     if (rows_per_item != 64) return -1;
@@ -647,18 +667,23 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     const float cap_scale = softcap > 0.f ? scale / softcap : 0.f;
     if (page_size >= 8 && (page_size & (page_size - 1)) == 0 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
 #define LAUNCH_DMA(HD)                                                                                              \
-    paged_attention_prefill_dma_kernel<HD><<<num_items, kPrefillThreads, 0, stream>>>(                              \
+    if (split_weights) LAUNCH_DMA_S(HD, true); else LAUNCH_DMA_S(HD, false)
+#define LAUNCH_DMA_S(HD, S)                                                                                         \
+    paged_attention_prefill_dma_kernel<HD, S><<<num_items, kPrefillThreads, 0, stream>>>(                           \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
         scale_log2e, window, q_stride, cap_scale, softcap)
-        if (head_dim == 64) LAUNCH_DMA(64);
-        else if (head_dim == 128) LAUNCH_DMA(128);
-        else LAUNCH_DMA(256);
+        if (head_dim == 64) { LAUNCH_DMA(64); }
+        else if (head_dim == 128) { LAUNCH_DMA(128); }
+        else { LAUNCH_DMA(256); }
 #undef LAUNCH_DMA
+#undef LAUNCH_DMA_S
         return launch_status();
     }
 #define LAUNCH_RTW(HD, RTW)                                                                                         \
-    paged_attention_prefill_kernel<HD, RTW><<<num_items, kPrefillThreads, 0, stream>>>(                             \
+    if (split_weights) LAUNCH_RTW_S(HD, RTW, true); else LAUNCH_RTW_S(HD, RTW, false)
+#define LAUNCH_RTW_S(HD, RTW, S)                                                                                    \
+    paged_attention_prefill_kernel<HD, RTW, S><<<num_items, kPrefillThreads, 0, stream>>>(                          \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
         scale_log2e, window, q_stride, cap_scale, softcap)
@@ -676,5 +701,6 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     }
 #undef LAUNCH
 #undef LAUNCH_RTW
+#undef LAUNCH_RTW_S
     return launch_status();
 }

@@ -126,6 +126,18 @@ __device__ __forceinline__ float capped_score(float score, float cap) {
     return cap > 0.f ? cap * tanhf(score / cap) : score;
 }
 
+// The same for the kernels whose operands are bfloat16 anyway: tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1) with the
+// hardware's exponential and reciprocal, exact to about 1e-7 of the cap (an infinite exponential gives 1).
+__device__ __forceinline__ float capped_score_fast(float scaled_over_cap, float cap) {
+    const float t = __builtin_amdgcn_exp2f(scaled_over_cap * 2.8853900817779268f);
+    return cap * (1.f - 2.f * __builtin_amdgcn_rcpf(t + 1.f));
+}
+
+// What the rounding of a softmax weight to bfloat16 leaves out.  The matrix cores take bfloat16 operands; a
+// kernel that is to weigh the values with float32 weights multiplies them by the rounded weight and by this
+// remainder (rounded in its turn) and adds both: 16 bits of the weight instead of 8.
+__device__ __forceinline__ float bf16_remainder(float p) { return p - to_float(from_float<bf16>(p)); }
+
 // The activations of a gated feed-forward, by the number the host passes (the table `ACTIVATIONS` of
 // the Python side holds the same numbers): every kernel that applies one goes through `activate`,
 // so a new activation is one line here, one there, and a case in `WLLM_BY_ACTIVATION`.

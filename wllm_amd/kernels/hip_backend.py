@@ -46,7 +46,7 @@ _SIGNATURES = {
     "wllm_paged_attention_generic_chunk_keys": [],
     "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                  c_int, c_int, c_float, c_void_p],
+                                  c_int, c_int, c_float, c_int, c_void_p],
     "wllm_paged_attention_mfma_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                       c_float, c_void_p],
@@ -55,7 +55,7 @@ _SIGNATURES = {
                                          c_int, c_float, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                     c_int, c_float, c_void_p],
+                                     c_int, c_float, c_int, c_void_p],
     "wllm_gemm_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_split_sum": [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -234,7 +234,7 @@ class HipBackend:
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
-                        plan=None, softcap=0.0):
+                        plan=None, softcap=0.0, exact_weights=False):
         self._on_gpu(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out)
         q_stride = qkv.shape[1]         # a row begins with the query heads; this many elements lie between two rows
         if plan is not None:
@@ -262,8 +262,8 @@ class HipBackend:
                     plan.prefill_rows,
                     _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(plan.partial_o),
                     _ptr(plan.partial_ml), num_heads, num_kv_heads,
-                    head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, self._stream()),
-                    "paged_attention (prompt portions, matrix cores)")
+                    head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, int(exact_weights),
+                    self._stream()), "paged_attention (prompt portions, matrix cores)")
             if plan.num_items == 0 and plan.num_reduce == 0:
                 return
             self._check(self.lib.wllm_paged_attention_mfma(
@@ -271,7 +271,8 @@ class HipBackend:
                 _ptr(plan.live_items), plan.num_items, _ptr(plan.reduce_items),
                 plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
                 _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                block_tables.shape[1], scale, window, q_stride, softcap, self._stream()), "paged_attention (matrix cores)")
+                block_tables.shape[1], scale, window, q_stride, softcap, int(exact_weights), self._stream()),
+                "paged_attention (matrix cores)")
             return
         if head_dim % 4 or head_dim > 256:
             raise KernelError(f"paged_attention: head_dim {head_dim} is not a multiple of 4 up to 256")

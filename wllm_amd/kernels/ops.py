@@ -303,7 +303,8 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
                     token_segment: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
                     seg_ctx_len: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                     head_dim: int, page_size: int, scale: float, window: int = 0,
-                    max_q_len: int = 0, max_ctx_len: int = 0, plan=None, softcap: float = 0.0) -> None:
+                    max_q_len: int = 0, max_ctx_len: int = 0, plan=None, softcap: float = 0.0,
+                    exact_weights: bool = False) -> None:
     """Softmax attention of every query over the keys of its own request in the paged cache.
 
     The batch is a row of segments; segment s holds tokens seg_q_start[s] .. +seg_q_len[s],
@@ -312,6 +313,10 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     max(0, p - window + 1) .. p (window 0: from key 0).  Query head h uses key/value head
     h // (num_heads // num_kv_heads).  Scores are scaled by `scale` and then, with `softcap` c > 0,
     bent to c * tanh(score / c); scores, softmax and the weighted sum accumulate in float32.
+    The bfloat16 matrix-core kernels round a softmax weight to bfloat16 before they multiply it with the
+    values; with `exact_weights` they carry what the rounding left out through a second product, so the
+    weights count with 16 bits (2^-17 of a weight, where float32 leaves 2^-24 and the values' own
+    rounding 2^-9).  The other kernels weigh in float32 either way.
     qkv T [n, width]: a row begins with the num_heads query heads, which is all that is read of it
     (the row of `rope_and_cache_write`, or any wider one); block_tables int32 [S, max_pages];
     out T [n, num_heads*head_dim].
@@ -339,7 +344,9 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     if n:
         backend().paged_attention(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len,
                                   out, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
-                                  int(max_q_len), int(max_ctx_len), plan, **({"softcap": float(softcap)} if softcap else {}))
+                                  int(max_q_len), int(max_ctx_len), plan,
+                                  **({"softcap": float(softcap)} if softcap else {}),
+                                  **({"exact_weights": True} if exact_weights else {}))
 
 
 def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,

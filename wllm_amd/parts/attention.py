@@ -191,7 +191,7 @@ class PagedAttention:
             ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
-            plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0)
+            plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0, exact_weights=s.weights_in_float32)
         if s.gate_weight:
             # the gate's columns lie behind the heads in the projected row
             gate = qkv[:, self.gate_offset:self.gate_offset + s.num_heads * s.head_dim]

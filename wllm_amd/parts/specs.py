@@ -55,7 +55,8 @@ class AttentionSpec(MixerSpec):
     `values_are_keys`: there is no value projection; a key head as projected (with its bias,
     before rotation and norm) is also the value head.  `gate_weight`: the concatenated heads are
     multiplied by sigmoid(W_gate h) before the output projection.  `o_bias`: a bias of the output
-    projection."""
+    projection.  `weights_in_float32`: the softmax weights are not rounded to the values' type before
+    they weigh the values (a design that wants its attention weights in 32-bit)."""
     kind: str = "attention"
     hidden_size: int = 0
     num_heads: int = 0
@@ -76,6 +77,7 @@ class AttentionSpec(MixerSpec):
     values_are_keys: bool = False
     gate_weight: Optional[str] = None
     o_bias: Optional[str] = None
+    weights_in_float32: bool = False
 
 
 @dataclass(frozen=True)
