@@ -172,7 +172,7 @@ class EmulatedKernels:
         return None
 
     def head_prepare(self, rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim, page_size,
-                     interleaved, norm_eps, values_are_keys, parts):
+                     interleaved, norm_eps, values_are_keys, parts, norm_dim=None):
         self._count("head_prepare")
         n, width = rows.shape
         if parts is not None:
@@ -201,7 +201,7 @@ class EmulatedKernels:
                 heads[..., :half] = x1 * cos - x2 * sin
                 heads[..., half:2 * half] = x2 * cos + x1 * sin
         if norm_eps is not None:
-            heads = heads * torch.rsqrt(heads.pow(2).mean(-1, keepdim=True) + norm_eps)
+            heads = heads * torch.rsqrt(heads.pow(2).sum(-1, keepdim=True) / (norm_dim or head_dim) + norm_eps)
         v[:, :r * head_dim] = heads.reshape(n, -1)
         rows.copy_(v.to(rows.dtype))
         if cache is not None:

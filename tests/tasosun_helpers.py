@@ -65,11 +65,45 @@ WIDE = dict(page_size=4, seed=8, std=0.06, norm_std=0.1, config=config(120, 80, 
     layer(attention(2, 1, 160, rot=(160, 50000.0, 3.0), window=130, scale=0.2), 56),
 ], loop=(1, 1, 4), eps=1e-4, emb=2.0))
 
-CONFIGS = {"mixed": MIXED, "odd": ODD, "sharp": SHARP, "wide": WIDE}
+# Heads of 6 and 10 elements (no multiple of four: the engine pads them), an odd width and vocabulary, every
+# size 1 that can be (one head, one layer in the loop, a loop of one time).
+SMALL = dict(page_size=16, seed=9, std=0.15, norm_std=0.1, config=config(53, 30, [
+    layer(attention(1, 1, 6, rot=(4, 20.0, 1.0), window=5, softcap=9.0, scale=1.1), 22),
+    layer(attention(4, 2, 10, rot=(10, 900.0, 16.0), window=64, softcap=11.0, scale=0.8), 34),
+], loop=(1, 2, 1), eps=1e-6, emb=1.0))
+
+CONFIGS = {"mixed": MIXED, "odd": ODD, "sharp": SHARP, "wide": WIDE, "small": SMALL}
 
 
-def write_folder(name: str, folder: str) -> str:
-    c = CONFIGS[name]
+def random_config(seed: int) -> dict:
+    """A configuration drawn at random from what the design allows: sizes, head counts, order and sizes of the
+    layers, windows, constants, the loop."""
+    import random
+    r = random.Random(seed)
+    width = r.choice([24, 32, 48, 64, 72, 96, 128, 160])
+    layers = []
+    for _ in range(r.randint(1, 4)):
+        kv = r.choice([1, 1, 2, 3, 4])
+        heads = kv * r.choice([1, 1, 2, 3, 4, 8])
+        dim = r.choice([6, 8, 12, 16, 20, 24, 32, 32, 40, 48, 64, 64, 96, 128])
+        rot = None if r.random() < 0.1 else (2 * r.randint(1, dim // 2), r.choice([100.0, 10000.0, 1e6]), r.choice([1.0, 2.0, 8.0, 32.0]))
+        window = None if r.random() < 0.1 else r.choice([1, 2, 5, 16, 17, 31, 32, 33, 64, 80, 200])
+        softcap = None if r.random() < 0.1 else r.choice([5.0, 15.0, 30.0, 50.0])
+        scale = dim ** -0.5 * r.choice([0.5, 1.0, 1.0, 4.0, 12.0])
+        layers.append(layer(attention(heads, kv, dim, rot=rot, window=window, softcap=softcap, scale=scale),
+                            None if r.random() < 0.2 else r.choice([24, 64, 100, 192, 256])))
+    loop = None
+    if r.random() < 0.8:
+        start = r.randint(0, len(layers))
+        stop = r.randint(start, len(layers))
+        loop = (start, stop, r.randint(1, 3))
+    return dict(page_size=16, seed=seed, std=r.choice([0.05, 0.1, 0.2]), norm_std=0.1,
+                config=config(r.choice([50, 97, 256, 300, 1000]), width, layers, loop=loop, eps=r.choice([1e-6, 1e-5]),
+                              emb=r.choice([0.5, 1.0, 3.0, 8.0])))
+
+
+def write_folder(name, folder: str) -> str:
+    c = CONFIGS[name] if isinstance(name, str) else name
     return write_random_model_from_config_json(folder, copy.deepcopy(c["config"]), c["seed"], std=c["std"],
                                                norm_std=c["norm_std"])
 
@@ -79,9 +113,10 @@ def random_ids(seed: int, length: int, vocab: int) -> list:
     return torch.randint(0, vocab, (length,), generator=g).tolist()
 
 
-def requests_for(name: str, lengths) -> dict:
-    vocab = CONFIGS[name]["config"]["vocab"]
-    return {f"q{i}": random_ids(1000 * i + len(name), n, vocab) for i, n in enumerate(lengths)}
+def requests_for(name, lengths) -> dict:
+    vocab = (CONFIGS[name] if isinstance(name, str) else name)["config"]["vocab"]
+    salt = len(name) if isinstance(name, str) else 3
+    return {f"q{i}": random_ids(1000 * i + salt, n, vocab) for i, n in enumerate(lengths)}
 
 
 def plain_logits(folder: str, requests: dict, dtype=torch.float64, round_to=None) -> dict:

@@ -18,7 +18,7 @@ from wllm_amd.engine.replay import TraceReplayer, pages_for_max_tokens
 from wllm_amd.kernels import ops
 from wllm_amd.parts import build_model, load_model
 
-LENGTHS = {"mixed": [70, 45, 90, 33, 58], "odd": [40, 66, 25, 51], "sharp": [80, 37, 64, 50], "wide": [30, 140, 21]}
+LENGTHS = {"mixed": [70, 45, 90, 33, 58], "odd": [40, 66, 25, 51], "sharp": [80, 37, 64, 50], "wide": [30, 140, 21], "small": [75, 20, 130]}
 FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions, "mixed": trace_mixed}
 
 

@@ -24,7 +24,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 DTYPES = [torch.float32, torch.bfloat16]
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LENGTHS = {"mixed": [70, 45, 150, 33, 58], "odd": [40, 66, 25, 151], "sharp": [80, 137, 64, 50], "wide": [30, 140, 21]}
+LENGTHS = {"mixed": [70, 45, 150, 33, 58], "odd": [40, 66, 25, 151], "sharp": [80, 137, 64, 50], "wide": [30, 140, 21], "small": [75, 20, 130]}
 FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions, "mixed": trace_mixed}
 
 
@@ -255,6 +255,26 @@ def test_replay_matches_plain(folders, name, family, dtype):
     assert all(g.pool.num_free == g.pool.num_pages for g in runner.cache.groups)
     exact, rounded = _references(folders[name], requests, dtype)
     compare_rows(got, exact, rounded, float32_relative=5e-5)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Other sizes, head counts, orders of layers, windows, constants and loops than any fixed case: a mixed trace
+    (portions beside decoded tokens, pages used again) in both precisions against the plain implementation."""
+    from tasosun_helpers import random_config
+    case = random_config(seed)
+    folder = write_folder(case, str(tmp_path / "m"))
+    requests = requests_for(case, [90, 41, 130, 23])
+    trace = trace_mixed(requests, seed=seed)
+    for dtype in ("float32", "bfloat16"):
+        model = load_model(folder, dtype, DEV)
+        runner = ModelRunner.create(model, num_pages=pages_for_max_tokens(max_live_tokens(trace), 16), page_size=16,
+                                    max_requests=4, poison_freed_pages=True)
+        with torch.inference_mode():
+            got = replay_and_collect(TraceReplayer(runner), trace)
+        runner.cache.check()
+        exact, rounded = _references(folder, requests, dtype)
+        compare_rows(got, exact, rounded, float32_relative=5e-5)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

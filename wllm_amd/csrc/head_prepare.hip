@@ -21,7 +21,8 @@ template <typename T> struct alignas(4 * sizeof(T)) Four { T v[4]; };
 //   2. where the values are the keys, the key head as it is now goes to the cache's values;
 //   3. the first rotary_dim elements turn by position * inv_freq[j]: pair j is (2j, 2j + 1)
 //      (interleaved) or (j, j + rotary_dim / 2);
-//   4. with norm_eps >= 0 the head is divided by sqrt(mean of its squares + norm_eps);
+//   4. with norm_eps >= 0 the head is divided by sqrt(sum of its squares / norm_dim + norm_eps) (norm_dim is
+//      head_dim, or less where the last elements of a head are padding that is always zero);
 //   5. it is written back to the row, and a key head to the cache's keys.
 // Value heads of their own and the rest of the row take step 1 only.  Keys lie in the cache as
 // [page_size, head_dim], values transposed as [head_dim, page_size].
@@ -39,7 +40,7 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
                     const float* __restrict__ bias, int bias_width, const int* __restrict__ positions,
                     const float* __restrict__ inv_freq, const int* __restrict__ slots, T* __restrict__ cache,
                     long long num_pages, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
-                    int interleaved, float norm_eps, int values_are_keys, int page_size, int head_pieces) {
+                    int interleaved, float norm_eps, int norm_dim, int values_are_keys, int page_size, int head_pieces) {
     __shared__ float staged[kPrepareWaves][FOUR ? 1 : kPrepareMaxHead];
     const int token = blockIdx.x;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -143,7 +144,7 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
         float inv = 1.f;
         if (norm_eps >= 0.f) {
             const float ss = wave_sum(v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3]);
-            inv = rsqrtf(ss / static_cast<float>(head_dim) + norm_eps);
+            inv = rsqrtf(ss / static_cast<float>(norm_dim) + norm_eps);
         }
         if (live) {
             Four<T> r;
@@ -186,7 +187,7 @@ head_prepare_kernel(T* __restrict__ rows, int row_width, const float* __restrict
         ss += v[k] * v[k];
     }
     float inv = 1.f;
-    if (norm_eps >= 0.f) inv = rsqrtf(wave_sum(ss) / static_cast<float>(head_dim) + norm_eps);
+    if (norm_eps >= 0.f) inv = rsqrtf(wave_sum(ss) / static_cast<float>(norm_dim) + norm_eps);
 #pragma unroll
     for (int k = 0; k < kPerLane; ++k) {
         const int e = lane + k * kWave;
@@ -204,11 +205,11 @@ WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const flo
                                long long split_stride, const float* bias, int bias_width, const int* positions,
                                const float* inv_freq, const int* slots, void* cache, long long num_pages, int n,
                                int num_heads, int num_kv_heads, int head_dim, int rotary_dim, int interleaved,
-                               float norm_eps, int values_are_keys, int page_size, hipStream_t stream) {
+                               float norm_eps, int norm_dim, int values_are_keys, int page_size, hipStream_t stream) {
     const int heads = num_heads + (values_are_keys ? 1 : 2) * num_kv_heads;
     if (head_dim <= 0 || head_dim > kPrepareMaxHead || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 != 0 ||
         row_width < heads * head_dim || num_heads < 0 || num_kv_heads < 0 || page_size <= 0 || bias_width < 0 ||
-        bias_width > row_width || (bias == nullptr && bias_width != 0))
+        bias_width > row_width || (bias == nullptr && bias_width != 0) || norm_dim <= 0 || norm_dim > head_dim)
         return -1;
     if (inv_freq == nullptr && rotary_dim != 0) return -1;
     if (n <= 0) return 0;
@@ -227,7 +228,7 @@ WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const flo
     head_prepare_kernel<T, FOUR><<<grid, kWave * kPrepareWaves, 0, stream>>>(                                       \
         static_cast<T*>(rows), row_width, parts, splits, static_cast<size_t>(split_stride), bias, bias_width, positions, \
         inv_freq, slots, static_cast<T*>(cache), num_pages, num_heads, num_kv_heads, head_dim, rotary_dim, interleaved, \
-        norm_eps, values_are_keys, page_size, head_pieces)
+        norm_eps, norm_dim, values_are_keys, page_size, head_pieces)
     if (is_bf16) {
         if (four) LAUNCH(bf16, true); else LAUNCH(bf16, false);
     } else {

@@ -353,7 +353,7 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
                  inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor], cache: Optional[torch.Tensor], *,
                  num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, interleaved: bool = False,
                  norm_eps: Optional[float] = None, values_are_keys: bool = False,
-                 parts: Optional[torch.Tensor] = None) -> None:
+                 parts: Optional[torch.Tensor] = None, norm_dim: Optional[int] = None) -> None:
     """What `rope_and_cache_write` does, for attention blocks that do more between projection and
     attention.  rows T [n, width]: num_heads query heads, num_kv_heads key heads, num_kv_heads value
     heads unless `values_are_keys`, then any further columns.  In this order, in float32: every
@@ -363,8 +363,9 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
     as it is now is stored as the value head; the first 2 * len(inv_freq) elements of every query
     and key head turn by position * inv_freq[j], pair j being elements (2j, 2j + 1) if
     `interleaved`, else (j, j + len(inv_freq)); with `norm_eps` every query and key head is
-    divided by sqrt(mean of its squares + norm_eps); the heads are written back and the key heads
-    stored.  slots, cache as in `rope_and_cache_write` (both None: nothing is stored)."""
+    divided by sqrt(sum of its squares / norm_dim + norm_eps) (norm_dim: head_dim unless given; less where
+    the last elements of every head are padding that is always zero); the heads are written back and the
+    key heads stored.  slots, cache as in `rope_and_cache_write` (both None: nothing is stored)."""
     heads = num_heads + (1 if values_are_keys else 2) * num_kv_heads
     _dense(rows, "rows", _ACT)
     _need(rows.dim() == 2 and rows.shape[1] >= heads * head_dim,
@@ -383,6 +384,8 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
         _need(inv_freq.dim() == 1 and 0 < 2 * inv_freq.shape[0] <= head_dim,
               lambda: f"inv_freq: {tuple(inv_freq.shape)} does not fit head_dim {head_dim}")
     _need(norm_eps is None or norm_eps >= 0.0, "norm_eps must not be negative")
+    norm_dim = head_dim if norm_dim is None else int(norm_dim)
+    _need(0 < norm_dim <= head_dim, "norm_dim: from 1 to head_dim")
     _need((slots is None) == (cache is None), "slots and cache go together")
     if cache is not None:
         _dense(slots, "slots", torch.int32, (n,))
@@ -391,7 +394,7 @@ def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: to
               lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
     if n:
         call("head_prepare", rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
-             page_size, bool(interleaved), norm_eps, bool(values_are_keys), parts)
+             page_size, bool(interleaved), norm_eps, bool(values_are_keys), parts, norm_dim)
 
 
 def _band(t: torch.Tensor, name: str, dtype, rows: int, cols: int) -> None:
@@ -693,17 +696,17 @@ def _register_own() -> None:
 
 
     def prepare(fn, stream, rows, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
-                page_size, interleaved, norm_eps, values_are_keys, parts):
+                page_size, interleaved, norm_eps, values_are_keys, parts, norm_dim):
         splits, stride = (parts.shape[0], parts.shape[1] * parts.shape[2]) if parts is not None else (0, 0)
         return fn(p(rows), int(rows.dtype == torch.bfloat16), rows.shape[1], p(parts), splits, stride, p(bias),
                   bias.shape[0] if bias is not None else 0, p(positions), p(inv_freq), p(slots), p(cache), cache.shape[0] if cache is not None else 0,
                   rows.shape[0], num_heads, num_kv_heads, head_dim,
                   2 * inv_freq.shape[0] if inv_freq is not None else 0, int(interleaved),
-                  float(norm_eps) if norm_eps is not None else -1.0, int(values_are_keys), page_size, stream)
+                  float(norm_eps) if norm_eps is not None else -1.0, norm_dim, int(values_are_keys), page_size, stream)
 
     register_op("head_prepare", entry_point="wllm_head_prepare",
                 argtypes=[c_void_p, c_int, c_int, c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                          c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                          c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
                 launch=prepare)
     register_op("sigmoid_gate", entry_point="wllm_sigmoid_gate",
                 argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_void_p],

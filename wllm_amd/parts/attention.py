@@ -39,7 +39,9 @@ class PagedAttention:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         if spec.window is not None and spec.window <= 0:
             raise ValueError(f"window must be positive or None, got {spec.window}")
-        if spec.head_dim % ops.HEAD_DIM_STEP or not 0 < spec.head_dim <= ops.MAX_HEAD_DIM:
+        plain = not (spec.softcap or spec.qk_norm_eps is not None or spec.values_are_keys or spec.gate_weight
+                     or spec.position.pairing == "interleaved")
+        if (plain and spec.head_dim % ops.HEAD_DIM_STEP) or not 0 < spec.head_dim <= ops.MAX_HEAD_DIM:
             raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of "
                              f"{ops.HEAD_DIM_STEP} up to {ops.MAX_HEAD_DIM}")
         if spec.values_are_keys and (spec.v_weight or spec.v_bias):
@@ -55,20 +57,24 @@ class PagedAttention:
         self.w_o = None
         self.b_o = None
         # the plain form runs the kernels that were written for it; anything else the general ones
-        self.plain = not (spec.softcap or spec.qk_norm_eps is not None or spec.values_are_keys or spec.gate_weight
-                          or getattr(self.position, "interleaved", False))
+        self.plain = plain
+        # The kernels take heads of a multiple of four elements.  A head of another size is padded at load with
+        # rows of zeros in its projections (and columns of zeros in the output projection): the padding is zero
+        # in queries, keys and values, adds nothing to a score or a result, and the unit norm divides by the
+        # true size.  Only the general path does this.
+        self.dim = spec.head_dim if plain else -(-spec.head_dim // ops.HEAD_DIM_STEP) * ops.HEAD_DIM_STEP
 
     @property
     def qkv_width(self) -> int:
         """Columns of the projected row: queries, keys, values (unless they are the keys), gate."""
         s = self.spec
         heads = s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads + (s.num_heads if s.gate_weight else 0)
-        return heads * s.head_dim
+        return heads * self.dim
 
     @property
     def gate_offset(self) -> int:
         s = self.spec
-        return (s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads) * s.head_dim
+        return (s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads) * self.dim
 
     def expected_tensors(self) -> dict:
         s = self.spec
@@ -92,9 +98,21 @@ class PagedAttention:
     def load(self, fetch) -> None:
         s = self.spec
         names = [s.q_weight, s.k_weight] + ([] if s.values_are_keys else [s.v_weight]) + ([s.gate_weight] if s.gate_weight else [])
-        w = torch.cat([fetch.matrix(name) for name in names], dim=0)
+        pad = self.dim - s.head_dim
+
+        def heads_padded(t: torch.Tensor, axis: int) -> torch.Tensor:
+            """`t` with every head of `axis` (heads * head_dim long) followed by `pad` zeros."""
+            if not pad:
+                return t
+            shape = list(t.shape)
+            heads = shape[axis] // s.head_dim
+            t = t.unflatten(axis, (heads, s.head_dim))
+            zeros = torch.zeros(shape[:axis] + [heads, pad] + shape[axis + 1:], dtype=t.dtype, device=t.device)
+            return torch.cat([t, zeros], dim=axis + 1).flatten(axis, axis + 1)
+
+        w = torch.cat([heads_padded(fetch.matrix(name), 0) for name in names], dim=0)
         self.w_qkv, self.t_qkv = load_matrix(fetch, w)        # the matrix and its tile-major copy
-        self.w_o, self.t_o = load_matrix(fetch, fetch.matrix(s.o_weight))
+        self.w_o, self.t_o = load_matrix(fetch, heads_padded(fetch.matrix(s.o_weight), 1))
         if s.o_bias is not None:
             self.b_o = fetch.to_device(fetch.vector(s.o_bias))
         if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
@@ -103,14 +121,15 @@ class PagedAttention:
             # (the gate's projection, behind the heads in the row, has none: the bias is shorter than the row)
             found = [fetch.vector(name) if name is not None else None for name, _ in biases]
             where = next(v.device for v in found if v is not None)      # a fetcher may make its tensors on the device
-            parts = [v if v is not None else torch.zeros(width, device=where) for v, (_, width) in zip(found, biases)]
+            parts = [heads_padded(v if v is not None else torch.zeros(width, device=where), 0)
+                     for v, (_, width) in zip(found, biases)]
             self.b_qkv = fetch.to_device(torch.cat(parts))
         if hasattr(self.position, "load"):
             self.position.load(fetch)
         self.position.prepare(fetch.device)
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+        return CacheNeed(self.spec.num_kv_heads, self.dim, self.spec.window)
 
     def state_shape(self):
         return None
@@ -126,7 +145,7 @@ class PagedAttention:
         layers of the shape; of fixed shape and rewritten in place in a captured graph."""
         s = self.spec
         # (the plan depends on these alone: layers that differ in their rows' width or cap share it)
-        shape = dict(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=page_size,
+        shape = dict(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=self.dim, page_size=page_size,
                      window=s.window or 0)
 
         def build(c):
@@ -161,9 +180,10 @@ class PagedAttention:
             projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
             ops.head_prepare(
                 qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage, num_heads=s.num_heads,
-                num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
+                num_kv_heads=s.num_kv_heads, head_dim=self.dim, page_size=pages.page_size,
                 interleaved=getattr(self.position, "interleaved", False), norm_eps=s.qk_norm_eps,
-                values_are_keys=s.values_are_keys, parts=projected if projected.dim() == 3 else None)
+                values_are_keys=s.values_are_keys, parts=projected if projected.dim() == 3 else None,
+                norm_dim=s.head_dim)
         elif apply is not None:
             ops.linear(h, self.w_qkv, qkv, self.t_qkv)
             if self.b_qkv is not None:
@@ -185,16 +205,16 @@ class PagedAttention:
                 qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage,
                 num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
                 parts=parts)
-        attn = ctx.buffer("attn", (n, s.num_heads * s.head_dim), h.dtype)
+        attn = ctx.buffer("attn", (n, s.num_heads * self.dim), h.dtype)
         ops.paged_attention(
             qkv, pages.storage, pages.block_tables, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
-            ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
+            ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=self.dim,
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
             plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0, exact_weights=s.weights_in_float32)
         if s.gate_weight:
             # the gate's columns lie behind the heads in the projected row
-            gate = qkv[:, self.gate_offset:self.gate_offset + s.num_heads * s.head_dim]
+            gate = qkv[:, self.gate_offset:self.gate_offset + s.num_heads * self.dim]
             target = product_input if product_input is not None else attn
             ops.sigmoid_gate(attn, gate, target)
             attn = target
