@@ -127,7 +127,7 @@ def cmd_bench_decode(args) -> int:
 
 
 def main(argv=None) -> int:
-    ap = argparse.ArgumentParser(prog="wllm_amd", description="Gemma inference engine for one MI355X")
+    ap = argparse.ArgumentParser(prog="wllm_amd", description="Inference engine for one MI355X (architectures: see wllm_amd.config.registered_architectures)")
     sub = ap.add_subparsers(dest="command", required=True)
 
     g = sub.add_parser("generate", help="generate token ids for prompts given as token ids")

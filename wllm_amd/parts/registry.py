@@ -4,7 +4,8 @@ A part is a class built from its specification alone.  It says which checkpoint
 tensors it expects, loads them, and runs on the flat batch of a step.  The
 interfaces:
 
-norm          expected_tensors(); load(fetch); forward(x, out, delta=None, rows=None)
+norm          expected_tensors(); load(fetch); forward(x, out, delta=None, rows=None[, delta_bias=None]):
+              `delta_bias` is passed only when a pending product brought a bias with it
 position      prepare(device); `inv_freq`: float32 [rotary_dim / 2] that the mixer's rotation kernels
               turn queries and keys by, or None; optionally `apply(ctx, qkv, *, num_heads,
               num_kv_heads, head_dim)`, a step of its own on the projected rows [tokens,
@@ -12,7 +13,9 @@ position      prepare(device); `inv_freq`: float32 [rotary_dim / 2] that the mix
               are cached, for encodings that are no rotation; optionally `expected_tensors()`
               and `load(fetch)` for tensors of its own
 mixer         expected_tensors(); load(fetch); cache_need() -> CacheNeed | None;
-              state_shape() -> tuple | None; forward(ctx, entry, h) -> y
+              state_shape() -> tuple | None; forward(ctx, entry, h) -> y; a mixer that ends in a product
+              and keeps its weight as `w_o` may be asked by a parallel block for
+              forward(ctx, entry, h, product_input=band) and then writes the product's input there
 feed-forward  expected_tensors(); load(fetch); forward(ctx, h) -> y
 block         built from a BlockSpec and the parts above; forward(ctx, entry, stream)
 
