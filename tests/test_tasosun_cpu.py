@@ -67,7 +67,6 @@ def test_runs_of_a_file_without_a_loop_and_of_a_loop_that_is_empty():
     (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=7), "even"),
     (lambda c: c["layers"][0].update(type="scan"), "attention"),
     (lambda c: c["layers"][0]["mlp"].update(kind="experts"), "dense"),
-    (lambda c: c["layers"][0]["mixer"].update(sinks=4), "sinks"),
     (lambda c: c.update(loop={"start": 2, "stop": 1, "times": 2}), "loop"),
     (lambda c: c.pop("norm"), "norm"),
 ])
@@ -76,6 +75,17 @@ def test_a_file_that_the_design_does_not_cover_is_refused(change, words):
     change(raw)
     with pytest.raises(ConfigError, match=words):
         TasosunConfig.from_dict(raw)
+
+
+def test_a_key_that_is_not_read_is_named_in_a_warning():
+    from wllm_amd.architectures.tasosun_config import UnknownConfigKey
+    raw = copy.deepcopy(CONFIGS["mixed"]["config"])
+    raw["note"] = "drawn by hand"
+    raw["layers"][0]["mixer"]["sinks"] = 4
+    with pytest.warns(UnknownConfigKey) as caught:
+        cfg = TasosunConfig.from_dict(raw)
+    assert any("sinks" in str(w.message) for w in caught) and any("note" in str(w.message) for w in caught)
+    assert cfg.layers[0].attention.heads == 4
 
 
 def test_the_written_config_reads_back(folders):

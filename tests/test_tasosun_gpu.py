@@ -125,6 +125,8 @@ def _attention_problem(dtype, nh, nkv, d, ps, segs, seed, extra_columns):
     (4, 2, 32, 16, 24, 30.0, [(1, 100), (70, 70), (1, 24), (1, 25), (5, 200)]),      # matrix cores, decoded rows and blocks of 64
     (6, 2, 96, 16, 40, 20.0, [(1, 41), (130, 300)]),
     (2, 1, 64, 8, 0, 6.0, [(1, 300), (65, 65)]),                                     # a cap without a window
+    (2, 1, 256, 16, 50, 12.0, [(1, 130), (80, 200)]),                               # the largest head
+    (4, 4, 128, 16, 0, 10.0, [(1, 70), (100, 100), (3, 3)]),
     (3, 3, 20, 8, 7, 5.0, [(1, 50), (33, 40), (1, 7), (1, 8)]),                     # the kernel on the vector units
     (2, 2, 160, 4, 1, 15.0, [(1, 9), (20, 20)]),                                     # a window of one
 ])
@@ -363,3 +365,22 @@ def test_the_trace_runner_and_the_command_line(folders, tmp_path):
     last = torch.frombuffer(bytearray((out / "2.f32").read_bytes()), dtype=torch.float32).view(1, -1)
     assert not (out / "1.f32").exists()
     compare_rows({("a", 0): first[0], ("a", 29): first[1], ("a", 44): last[0]}, exact, float32_relative=5e-5)
+    # the command line: a model folder of a named shape, then greedy generation from it
+    made = tmp_path / "made"
+    r = subprocess.run([sys.executable, "-m", "wllm_amd.cli", "random-model", "--out", str(made), "--config", "tasosun-tiny",
+                        "--seed", "3", "--std", "0.3"], cwd=ROOT, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run([sys.executable, "-m", "wllm_amd.cli", "generate", "--model", str(made), "--dtype", "float32",
+                        "--prompt-ids", "5,17,3,200,41", "--max-new-tokens", "6"], cwd=ROOT, capture_output=True, text=True,
+                       timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads([x for x in r.stdout.splitlines() if x.startswith("{")][-1])
+    cfg, w = tasosun_plain.read_config(str(made)), tasosun_plain.read_weights(str(made), torch.float64)
+    tokens = [5, 17, 3, 200, 41]
+    for t in line["token_ids"]:
+        logits = tasosun_plain.forward(cfg, w, tokens)[-1]
+        if (logits.topk(2).values[0] - logits.topk(2).values[1]).item() < 1e-3:
+            break
+        assert t == int(logits.argmax())
+        tokens.append(t)
+    assert len(line["token_ids"]) == 6

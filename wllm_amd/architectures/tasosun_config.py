@@ -6,15 +6,21 @@ constants of its mixer under `mixer`, and its feed-forward under `mlp`, or null 
 `loop` (`start`, `stop`, `times`: the layers start .. stop-1 run `times` times in a row).
 Every layer carries its own sizes, so two layers of one model may differ in all of them.
 Nothing has a default that a model could rely on silently: a key the design needs and the
-file lacks is an error, and so is a key of a layer that this code does not know (an option
-that would be ignored is a model that computes something else).
+file lacks is an error.  A key that this code does not know is named in a warning
+(`UnknownConfigKey`) and otherwise ignored: it may be a note of whoever wrote the file, or an
+option of a later version of the design, which would then compute something else.
 """
 from __future__ import annotations
 
+import warnings
 from dataclasses import dataclass
 from typing import Optional
 
 from wllm_amd.config.registry import ConfigError
+
+
+class UnknownConfigKey(UserWarning):
+    """config.json holds a key that the implementation does not read."""
 
 
 def _positive_int(where: str, v) -> int:
@@ -37,7 +43,8 @@ def _section(where: str, raw, required: tuple, optional: tuple = ()) -> dict:
         raise ConfigError(f"{where} lacks required key(s): {', '.join(missing)}")
     unknown = sorted(set(raw) - set(required) - set(optional))
     if unknown:
-        raise ConfigError(f"{where} has key(s) this implementation does not know: {', '.join(unknown)}")
+        warnings.warn(f"{where} has key(s) this implementation does not read: {', '.join(unknown)}", UnknownConfigKey,
+                      stacklevel=3)
     return raw
 
 
