@@ -102,6 +102,27 @@ def random_config(seed: int) -> dict:
                               emb=r.choice([0.5, 1.0, 3.0, 8.0])))
 
 
+def middling_config(seed: int) -> dict:
+    """Layers of some hundred columns, windows of about a hundred keys, a loop: sizes at which a request of a
+    thousand tokens crosses many windows, pages and chunks of keys."""
+    import random
+    r = random.Random(1000 + seed)
+    width = r.choice([192, 256, 384, 512])
+    kinds = []
+    for _ in range(r.randint(1, 2)):        # one or two kinds of layer, repeated
+        kv = r.choice([1, 2, 4])
+        heads = kv * r.choice([1, 2, 3, 6, 12])
+        dim = r.choice([48, 64, 80, 112, 128])
+        kinds.append(layer(attention(heads, kv, dim, rot=(2 * r.randint(4, dim // 2), r.choice([10000.0, 500000.0]), r.choice([1.0, 4.0, 8.0])),
+                                     window=r.choice([64, 65, 100, 127, 128, 160]), softcap=r.choice([20.0, 50.0]),
+                                     scale=dim ** -0.5 * r.choice([1.0, 3.0])), r.choice([None, 256, 512, 640])))
+    layers = [copy.deepcopy(kinds[i % len(kinds)]) for i in range(r.randint(3, 6))]
+    start = r.randint(0, len(layers) - 1)
+    return dict(page_size=16, seed=seed, std=0.06, norm_std=0.1,
+                config=config(r.choice([300, 512, 777]), width, layers, loop=(start, r.randint(start + 1, len(layers)), r.randint(2, 3)),
+                              eps=1e-6, emb=r.choice([1.0, 3.0])))
+
+
 def write_folder(name, folder: str) -> str:
     c = CONFIGS[name] if isinstance(name, str) else name
     return write_random_model_from_config_json(folder, copy.deepcopy(c["config"]), c["seed"], std=c["std"],

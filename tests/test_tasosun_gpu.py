@@ -279,6 +279,32 @@ def test_configurations_drawn_at_random(tmp_path, seed):
         compare_rows(got, exact, rounded, float32_relative=5e-5)
 
 
+@pytest.mark.parametrize("seed", range(2))
+def test_long_requests_at_middling_sizes(tmp_path, seed):
+    """Requests of up to 1,100 tokens: whole, with a tail of 140 tokens decoded one by one (windows pass over
+    decoded tokens), and four live at a time in portions beside decoded tokens, in a pool made for what is
+    live; every 7th position is compared."""
+    from tasosun_helpers import middling_config
+    case = middling_config(seed)
+    folder = write_folder(case, str(tmp_path / "m"))
+    requests = requests_for(case, [1100, 400, 333, 90, 610])
+    thin = lambda trace: [dict(st, entries=[dict(e, want=[w for w in e["want"] if (w + len(e["tokens"])) % 7 == 0 or len(e["tokens"]) == 1])
+                                             for e in st["entries"]]) for st in trace]
+    one = {"q0": requests["q0"]}
+    traces = [thin(trace_whole(one)), thin(trace_tail(one, tail=140)),
+              thin(trace_mixed(requests, seed=seed, portion_sizes=(2, 16, 37, 64, 130)))]
+    for dtype in ("float32", "bfloat16"):
+        model = load_model(folder, dtype, DEV)
+        exact, rounded = _references(folder, requests, dtype)
+        for trace in traces:
+            runner = ModelRunner.create(model, num_pages=pages_for_max_tokens(max_live_tokens(trace), 16), page_size=16,
+                                        max_requests=4, poison_freed_pages=True)
+            with torch.inference_mode():
+                got = replay_and_collect(TraceReplayer(runner), trace)
+            runner.cache.check()
+            compare_rows(got, exact, rounded, float32_relative=5e-5)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_through_windows_in_a_small_pool(folders, dtype):
     """300 tokens decoded one by one after a short prompt, in a pool that only holds them because windows
