@@ -134,7 +134,7 @@ class EmulatedKernels:
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
-                        plan=None, softcap=0.0, exact_weights=False):
+                        plan=None, softcap=0.0, exact_weights=False, chunk=0, sinks=None):
         self._count("paged_attention")
         n = qkv.shape[0]
         n_rep = num_heads // num_kv_heads
@@ -158,13 +158,20 @@ class EmulatedKernels:
             allowed = key[None, :] <= pos[:, None]
             if window:
                 allowed &= key[None, :] > pos[:, None] - window
+            if chunk:
+                allowed &= key[None, :] >= (pos[:, None] // chunk) * chunk
             scores = torch.einsum("qhd,khd->hqk", q, k) * scale
             if softcap:
                 scores = softcap * torch.tanh(scores / softcap)
             # keys outside the window may hold NaN of pages given back: mask by selection, not by addition
             scores = torch.where(allowed[None], scores, torch.full_like(scores, float("-inf")))
-            probs = torch.softmax(scores, dim=-1)
-            v = torch.where(torch.isnan(v), torch.zeros_like(v), v) if window else v
+            if sinks is not None:
+                # one more term of the denominator: a column that is dropped after the softmax
+                sink = sinks.to(self.acc)[:, None, None].expand(-1, ql, 1)
+                probs = torch.softmax(torch.cat([scores, sink], dim=-1), dim=-1)[..., :-1]
+            else:
+                probs = torch.softmax(scores, dim=-1)
+            v = torch.where(torch.isnan(v), torch.zeros_like(v), v) if (window or chunk) else v
             o = torch.einsum("hqk,khd->qhd", probs, v)
             out[q0:q0 + ql] = o.reshape(ql, num_heads * head_dim).to(out.dtype)
 
@@ -217,9 +224,109 @@ class EmulatedKernels:
             kview[page, :, off, :] = k
             vview[page, :, :, off] = val
 
-    def sigmoid_gate(self, a, gate, out):
+    def sigmoid_gate(self, a, gate, out, per=1):
         self._count("sigmoid_gate")
-        out.copy_((a.to(self.acc) * torch.sigmoid(gate.to(self.acc))).to(out.dtype))
+        g = torch.sigmoid(gate.to(self.acc)).repeat_interleave(per, dim=1)
+        out.copy_((a.to(self.acc) * g).to(out.dtype))
+
+    # ---- the general norm step, the band norm, the token input's lookup, the product head by head ----
+    def _normed(self, v, recipe):
+        if recipe is None:
+            return v
+        if recipe.kind == "layer":
+            v = v - v.mean(-1, keepdim=True)
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + recipe.eps) * (recipe.offset + recipe.weight.to(self.acc))
+
+    def norm_add(self, x, delta, delta_norm, out, out_norm, rows):
+        self._count("norm_add")
+        idx = rows.long() if rows is not None else slice(None)
+        v = x[idx].to(self.acc)
+        if delta is not None:
+            if delta.dim() == 3:
+                total = delta[0]
+                for p in range(1, delta.shape[0]):
+                    total = total + delta[p]
+                delta = total
+            v = (v + self._normed(delta[idx].to(self.acc), delta_norm)).to(x.dtype)
+            if rows is None:
+                x.copy_(v)
+            v = v.to(self.acc)
+        if out is not None:
+            out.copy_(self._normed(v, out_norm).to(out.dtype))
+
+    def band_norm(self, bands, eps):
+        self._count("band_norm")
+        for src, weight, count, out in bands:
+            v = src.to(self.acc)
+            y = v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) / count + eps) * weight.to(self.acc)
+            cols = src.shape[1]
+            result = torch.zeros(out.shape, dtype=out.dtype, device=out.device)
+            result[:, :cols] = y.to(out.dtype)
+            out.copy_(result)
+
+    def gated_lookup(self, gate, ids, table, col0, out, activation):
+        self._count("gated_lookup")
+        z = gate.to(self.acc)
+        if activation == "gelu_tanh":
+            a = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+        else:
+            a = z * torch.sigmoid(z)
+        out.copy_((a * table[ids.long(), col0:col0 + gate.shape[1]].to(self.acc)).to(out.dtype))
+
+    def head_linear(self, x, w, y):
+        self._count("head_linear")
+        heads, o, k = w.shape
+        n = x.shape[0]
+        r = torch.einsum("nhk,hok->nho", x.reshape(n, heads, k).to(self.acc), w.to(self.acc))
+        y.copy_(r.reshape(n, heads * o).to(y.dtype))
+
+    # ---- the state-space mixer's three kernels ----
+    def causal_conv(self, inp, weight, bias, state, carried_offset, token_segment, seg_q_start, seg_q_len, state_slots, out):
+        self._count("causal_conv")
+        c, taps = weight.shape
+        for s in range(seg_q_start.shape[0]):
+            q0, ql, slot = int(seg_q_start[s]), int(seg_q_len[s]), int(state_slots[s])
+            if ql == 0:
+                continue
+            carried = state[slot, carried_offset:carried_offset + (taps - 1) * c].view(taps - 1, c)
+            seq = torch.cat([carried.to(self.acc), inp[q0:q0 + ql].to(self.acc)], dim=0)
+            acc = bias.to(self.acc).expand(ql, -1).clone()
+            for k in range(taps):
+                acc = acc + seq[k:k + ql] * weight[:, k].to(self.acc)
+            out[q0:q0 + ql] = (acc * torch.sigmoid(acc)).to(out.dtype)
+            if taps > 1:
+                carried.copy_(seq[ql:].to(torch.float32))
+
+    def ssm_scan(self, xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y, heads, groups,
+                 state_size, head_dim):
+        self._count("ssm_scan")
+        inner, n_s = heads * head_dim, state_size
+        per = heads // groups
+        a = -torch.exp(a_log.to(self.acc))
+        for s in range(seg_q_start.shape[0]):
+            q0, ql, slot = int(seg_q_start[s]), int(seg_q_len[s]), int(state_slots[s])
+            if ql == 0:
+                continue
+            S = state[slot, :heads * n_s * head_dim].view(heads, n_s, head_dim)
+            cur = S.to(self.acc)
+            for t in range(q0, q0 + ql):
+                x = xbc[t, :inner].to(self.acc).view(heads, head_dim)
+                b = xbc[t, inner:inner + groups * n_s].to(self.acc).view(groups, n_s).repeat_interleave(per, dim=0)
+                c = xbc[t, inner + groups * n_s:].to(self.acc).view(groups, n_s).repeat_interleave(per, dim=0)
+                step = torch.nn.functional.softplus(dt[t].to(self.acc) + dt_bias.to(self.acc), threshold=1e9)
+                cur = torch.exp(a * step)[:, None, None] * cur + step[:, None, None] * b[:, :, None] * x[:, None, :]
+                cur = cur.to(torch.float32).to(self.acc)        # the state lives in float32
+                yt = torch.einsum("hnp,hn->hp", cur, c) + d_skip.to(self.acc)[:, None] * x
+                y[t] = yt.reshape(inner).to(y.dtype)
+            S.copy_(cur.to(torch.float32))
+
+    def gated_group_norm(self, y, z, weight, out, groups, eps):
+        self._count("gated_group_norm")
+        n, w = y.shape
+        zz = z.to(self.acc)
+        v = (y.to(self.acc) * zz * torch.sigmoid(zz)).view(n, groups, w // groups)
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        out.copy_((v.reshape(n, w) * weight.to(self.acc)).to(out.dtype))
 
     def copy_columns(self, src, out):
         self._count("copy_columns")

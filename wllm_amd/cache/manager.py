@@ -46,10 +46,12 @@ class OutOfSlots(RuntimeError):
 class CacheNeed:
     """What one schedule entry keeps per token: keys and values of
     `num_kv_heads` heads of `head_dim`; all of them (window None) or the last
-    `window`.  Stored in the model's dtype."""
+    `window`, or (`chunk`) those of the newest chunk of `chunk` positions counted
+    from 0.  Stored in the model's dtype."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    chunk: Optional[int] = None
     dtype = None
 
     def page_shape(self, page_size: int) -> tuple:
@@ -187,6 +189,10 @@ class CacheManager:
         ps = self.page_size
         need = self.groups[group_index].need
         total = -(-num_tokens // ps)
+        chunk = getattr(need, "chunk", None)
+        if chunk is not None:
+            # a chunk's first key and the newest token of a portion can straddle pages
+            return min(total, -(-(chunk + longest_portion) // ps) + 1)
         if need.window is None:
             return total
         # a window's oldest key and the newest token of a portion can straddle pages
@@ -264,10 +270,14 @@ class CacheManager:
         rc = self.requests[request]
         rc.context_len += num_new_tokens
         for gi, g in enumerate(self.groups):
-            w = g.need.window
-            if w is None:
+            w, chunk = g.need.window, getattr(g.need, "chunk", None)
+            if w is None and chunk is None:
                 continue
-            first_needed = max(0, rc.context_len - w + 1) // self.page_size
+            if chunk is not None:
+                # the next query, at position context_len, reaches back to the start of its own chunk
+                first_needed = (rc.context_len - rc.context_len % chunk) // self.page_size
+            else:
+                first_needed = max(0, rc.context_len - w + 1) // self.page_size
             table = rc.tables[gi]
             while rc.first_live[gi] < min(first_needed, len(table)):
                 i = rc.first_live[gi]

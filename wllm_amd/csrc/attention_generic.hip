@@ -3,7 +3,8 @@
 // path and of sizes the matrix-core kernels refuse.
 //
 // A token at position p (from its segment: p = ctx_len - q_len + i) sees keys lo..p with
-// lo = max(0, p - window + 1).  The keys are cut into chunks of kChunkKeys keys counted from
+// lo = lowest_key(p, window): all keys, a sliding window, or the keys of p's own chunk of positions.
+// With `sinks` (one float32 a query head) the softmax's denominator holds exp(sink) once more.  The keys are cut into chunks of kChunkKeys keys counted from
 // key 0, so a chunk's boundaries depend on the key index alone.  One workgroup takes one
 // (token, key/value head, chunk); its eight wavefronts take 16 keys each, and a wavefront's
 // work is two trips to memory: the rows of its 16 keys (lane = key and quarter of the
@@ -62,12 +63,12 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
                                float* __restrict__ partial_o, float* __restrict__ partial_ml, int token_begin,
                                int max_chunks, int num_heads, int num_kv_heads, int head_dim, int page_size,
                                int max_pages, float scale, int window, int group_begin, int q_stride,
-                               float softcap) {
+                               float softcap, const float* __restrict__ sinks) {
     const int token = token_begin + blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
     const int seg = token_segment[token];
     const int q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
     const int pos = ctx - q_len + (token - seg_q_start[seg]);
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = lowest_key(pos, window);
     const int c_lo = lo / kChunkKeys, c_hi = min(pos / kChunkKeys, max_chunks - 1);   // the bound keeps every access inside the buffers
     if (chunk < c_lo || chunk > c_hi) return;
     // the caller's bound on the context lengths was below this token's: its keys beyond the bound are not
@@ -262,6 +263,8 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
             }
             if (cut_short) num = __builtin_nanf("");
             if (whole) {
+                // a sink: one more term of the denominator, exp(sink of the head), with no key and no value
+                if (sinks) den += expf(sinks[head0 + g] - mm);
                 orow[g * head_dim + d] = from_float<T>(num / den);
             } else {
                 const size_t row = part_row + g * part_stride;
@@ -284,11 +287,11 @@ paged_attention_generic_reduce_kernel(const float* __restrict__ partial_o, const
                                       const int* __restrict__ token_segment, const int* __restrict__ seg_q_start,
                                       const int* __restrict__ seg_q_len, const int* __restrict__ seg_ctx_len,
                                       T* __restrict__ out, int token_begin, int max_chunks, int num_heads, int head_dim,
-                                      int window) {
+                                      int window, const float* __restrict__ sinks) {
     const int token = token_begin + blockIdx.x, head = blockIdx.y;
     const int seg = token_segment[token];
     const int pos = seg_ctx_len[seg] - seg_q_len[seg] + (token - seg_q_start[seg]);
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = lowest_key(pos, window);
     const int c_lo = lo / kChunkKeys, c_hi = min(pos / kChunkKeys, max_chunks - 1);   // the bound keeps every access inside the buffers
     if (c_lo == c_hi) return;
     const size_t row0 = (static_cast<size_t>(blockIdx.x) * num_heads + head) * max_chunks;
@@ -302,6 +305,7 @@ paged_attention_generic_reduce_kernel(const float* __restrict__ partial_o, const
         num = fmaf(partial_o[(row0 + ch) * head_dim + d], f, num);
         den = fmaf(partial_ml[(row0 + ch) * 2 + 1], f, den);
     }
+    if (sinks) den += expf(sinks[head] - mm);
     out[(static_cast<size_t>(token) * num_heads + head) * head_dim + d] = from_float<T>(num / den);
 }
 
@@ -326,7 +330,7 @@ WLLM_API int wllm_paged_attention_generic(const void* qkv, const void* cache, in
                                           const int* seg_ctx_len, void* out, void* partial_o, void* partial_ml,
                                           int partial_tokens, int max_ctx_len, int n, int num_heads, int num_kv_heads,
                                           int head_dim, int page_size, int max_pages, float scale, int window,
-                                          int q_stride, float softcap, hipStream_t stream) {
+                                          int q_stride, float softcap, const float* sinks, hipStream_t stream) {
     if (q_stride < num_heads * head_dim || softcap < 0.f) return -1;
     if (head_dim <= 0 || head_dim % 4 != 0 || head_dim > kMaxHeadDim || num_heads % num_kv_heads != 0) return -1;
     if (partial_tokens < 1 || max_ctx_len < 1 || !partial_o || !partial_ml) return -1;
@@ -344,7 +348,7 @@ WLLM_API int wllm_paged_attention_generic(const void* qkv, const void* cache, in
     paged_attention_generic_kernel<T, NV, DPL, V4><<<grid, kWave * kWaves, smem, stream>>>(                              \
         static_cast<const T*>(qkv), static_cast<const T*>(cache), block_tables, token_segment, seg_q_start, seg_q_len,  \
         seg_ctx_len, static_cast<T*>(out), static_cast<float*>(partial_o), static_cast<float*>(partial_ml), t0,         \
-        max_chunks, num_heads, num_kv_heads, head_dim, page_size, max_pages, scale, window, gb, q_stride, softcap)
+        max_chunks, num_heads, num_kv_heads, head_dim, page_size, max_pages, scale, window, gb, q_stride, softcap, sinks)
 #define LAUNCH_SIZES(T, V4)                         \
     if (nv == 4) LAUNCH(T, 4, 1, V4);               \
     else if (nv == 8) LAUNCH(T, 8, 2, V4);          \
@@ -363,11 +367,11 @@ WLLM_API int wllm_paged_attention_generic(const void* qkv, const void* cache, in
             if (is_bf16)
                 paged_attention_generic_reduce_kernel<bf16><<<rgrid, kMaxHeadDim, 0, stream>>>(
                     static_cast<const float*>(partial_o), static_cast<const float*>(partial_ml), token_segment, seg_q_start,
-                    seg_q_len, seg_ctx_len, static_cast<bf16*>(out), t0, max_chunks, num_heads, head_dim, window);
+                    seg_q_len, seg_ctx_len, static_cast<bf16*>(out), t0, max_chunks, num_heads, head_dim, window, sinks);
             else
                 paged_attention_generic_reduce_kernel<float><<<rgrid, kMaxHeadDim, 0, stream>>>(
                     static_cast<const float*>(partial_o), static_cast<const float*>(partial_ml), token_segment, seg_q_start,
-                    seg_q_len, seg_ctx_len, static_cast<float*>(out), t0, max_chunks, num_heads, head_dim, window);
+                    seg_q_len, seg_ctx_len, static_cast<float*>(out), t0, max_chunks, num_heads, head_dim, window, sinks);
             if (const int err = launch_status()) return err;
         }
     }

@@ -103,13 +103,13 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     const int width = q_stride;                     // elements between two tokens' query rows
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
-    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
+    const int seg_lo = lowest_key(first_pos, window);   // keys below may be given back
     const int row = row_begin + i;
     const bool row_valid = row < total_rows;
     const int tok = row_valid ? row / group : 0;
     const int head = kvh * group + (row_valid ? row % group : 0);
     const int pos = first_pos + tok;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = lowest_key(pos, window);
     // An item's keys lie within one aligned group of 128 (the host's chunk), so each of the four
     // wavefronts has at most one block of 32 keys and nothing is carried from block to block.
     const int blk_first = key_begin / kKeysPerBlock;

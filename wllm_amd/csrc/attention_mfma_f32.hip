@@ -63,13 +63,13 @@ paged_attention_f32_kernel(const float* __restrict__ qkv, const float* __restric
     const int width = q_stride;         // elements between two tokens' query rows
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
-    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
+    const int seg_lo = lowest_key(first_pos, window);   // keys below may be given back
     const int row = row_begin + i;
     const bool row_valid = row < total_rows;
     const int tok = row_valid ? row / group : 0;
     const int head = kvh * group + (row_valid ? row % group : 0);
     const int pos = first_pos + tok;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = lowest_key(pos, window);
     const int blk_first = key_begin / kKeysPerBlock;
     const int blk_end = (key_end + kKeysPerBlock - 1) / kKeysPerBlock;
     const int blk = blk_first + wave;
@@ -335,7 +335,7 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
     const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
-    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int seg_lo = lowest_key(first_pos, window);
     const int width = q_stride;         // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
@@ -348,17 +348,17 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
     const int tok = row_valid ? row / group : 0;
     const int head = kvh * group + (row_valid ? row % group : 0);
     const int pos = first_pos + tok;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = lowest_key(pos, window);
     // a block that lies wholly inside every row's range needs no mask (a wavefront-wide decision)
     const int w_last_row = min(total_rows - 1, wr0 + 15);
     const bool wave_active = wr0 < total_rows;
     const int t_pos_min = (wave_active && w_last_row == wr0 + 15) ? first_pos + wr0 / group : -1;
-    const int t_lo_max = window > 0 ? max(0, first_pos + max(w_last_row, 0) / group - window + 1) : 0;
+    const int t_lo_max = lowest_key(first_pos + max(w_last_row, 0) / group, window);
     const int w_hi = wave_active ? first_pos + w_last_row / group + 1 : 0;                       // exclusive
-    const int w_lo = window > 0 ? max(0, first_pos + wr0 / group - window + 1) : 0;
+    const int w_lo = lowest_key(first_pos + wr0 / group, window);
     const int b_last_row = min(total_rows - 1, row_begin + 63);
     const int b_hi = first_pos + b_last_row / group + 1;
-    const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
+    const int b_lo = lowest_key(first_pos + row_begin / group, window);
     const int blk_first = max(b_lo, key_begin) / kBlockKeys;
     const int blk_end = (min(b_hi, key_end) + kBlockKeys - 1) / kBlockKeys;
 

@@ -70,7 +70,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
     const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
-    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int seg_lo = lowest_key(first_pos, window);
     const int width = q_stride;         // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
@@ -89,7 +89,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
         tok[rt] = row_valid[rt] ? row[rt] / group : 0;
         head[rt] = kvh * group + (row_valid[rt] ? row[rt] % group : 0);
         pos[rt] = first_pos + tok[rt];
-        lo[rt] = window > 0 ? max(0, pos[rt] - window + 1) : 0;
+        lo[rt] = lowest_key(pos[rt], window);
         const bf16* qrow = qkv + static_cast<size_t>(q_start + tok[rt]) * width + static_cast<size_t>(head[rt]) * HD;
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
@@ -105,18 +105,18 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
         const int first = wr0 + rt * 16, last = min(total_rows - 1, first + 15);
         t_pos_min[rt] = first < total_rows ? first_pos + first / group : -1;
         const int pmax = first_pos + max(last, 0) / group;
-        t_lo_max[rt] = window > 0 ? max(0, pmax - window + 1) : 0;
+        t_lo_max[rt] = lowest_key(pmax, window);
         if (last < first + 15) t_pos_min[rt] = -1;      // a tile with rows beyond the segment always masks
     }
     // keys the wavefront's rows can need
     const bool wave_active = wr0 < total_rows;
     const int w_last_row = min(total_rows - 1, wr0 + kWaveRows - 1);
     const int w_hi = wave_active ? first_pos + w_last_row / group + 1 : 0;                       // exclusive
-    const int w_lo = window > 0 ? max(0, first_pos + wr0 / group - window + 1) : 0;
+    const int w_lo = lowest_key(first_pos + wr0 / group, window);
     // keys the workgroup stages: from the first wavefront's lowest to the last row's highest
     const int b_last_row = min(total_rows - 1, row_begin + kPrefillRows - 1);
     const int b_hi = first_pos + b_last_row / group + 1;
-    const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
+    const int b_lo = lowest_key(first_pos + row_begin / group, window);
     const int blk_first = max(b_lo, key_begin) / kBlockKeys;
     const int blk_end = (min(b_hi, key_end) + kBlockKeys - 1) / kBlockKeys;
     // the pages of keys blk_first * 32 .. blk_end * 32 (clamped to the request's keys)
@@ -406,7 +406,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
     const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
-    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int seg_lo = lowest_key(first_pos, window);
     const int width = q_stride;         // elements between two tokens' query rows
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
@@ -419,7 +419,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
     const int tok = row_valid ? row / group : 0;
     const int head = kvh * group + (row_valid ? row % group : 0);
     const int pos = first_pos + tok;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo = lowest_key(pos, window);
     bf16x8_t qreg[DC];
     {
         const bf16* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD;
@@ -436,16 +436,16 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
         const int last = min(total_rows - 1, wr0 + 15);
         t_pos_min = wr0 < total_rows ? first_pos + wr0 / group : -1;
         const int pmax = first_pos + max(last, 0) / group;
-        t_lo_max = window > 0 ? max(0, pmax - window + 1) : 0;
+        t_lo_max = lowest_key(pmax, window);
         if (last < wr0 + 15) t_pos_min = -1;      // a tile with rows beyond the segment always masks
     }
     const bool wave_active = wr0 < total_rows;
     const int w_last_row = min(total_rows - 1, wr0 + 15);
     const int w_hi = wave_active ? first_pos + w_last_row / group + 1 : 0;                       // exclusive
-    const int w_lo = window > 0 ? max(0, first_pos + wr0 / group - window + 1) : 0;
+    const int w_lo = lowest_key(first_pos + wr0 / group, window);
     const int b_last_row = min(total_rows - 1, row_begin + kPrefillRows - 1);
     const int b_hi = first_pos + b_last_row / group + 1;
-    const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
+    const int b_lo = lowest_key(first_pos + row_begin / group, window);
     const int blk_first = max(b_lo, key_begin) / kBlockKeys;
     const int blk_end = (min(b_hi, key_end) + kBlockKeys - 1) / kBlockKeys;
     const int page_base = blk_first * kBlockKeys / page_size;

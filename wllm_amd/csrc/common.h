@@ -114,6 +114,16 @@ __device__ __forceinline__ float stack_sum(const float* __restrict__ p, int spli
     return total;
 }
 
+// The lowest key a query at position `pos` sees, from the one integer every attention kernel takes as
+// its mask: 0, all keys from 0; w > 0, a sliding window of w keys (pos - w + 1, not below 0); -c < 0,
+// chunks of c positions counted from 0 (the first position of pos's own chunk).  It never falls as
+// pos rises, which is all the kernels' bounds over blocks of rows rely on.
+__host__ __device__ __forceinline__ int lowest_key(int pos, int window) {
+    if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+    if (window < 0) return pos - pos % (-window);
+    return 0;
+}
+
 // 2^x by the hardware instruction alone, for the arguments of a softmax (x <= 0, -inf included):
 // results below the smallest normal number become 0 instead of passing through the library's
 // rescaling, which a probability does not need.

@@ -244,7 +244,7 @@ WLLM_API int wllm_head_prepare(void* rows, int is_bf16, int row_width, const flo
 template <typename T, bool FOUR>
 __global__ void sigmoid_gate_kernel(const T* __restrict__ a, long long a_stride, const T* __restrict__ gate,
                                     long long gate_stride, T* __restrict__ out, long long out_stride, int rows,
-                                    int cols) {
+                                    int cols, int per) {
     constexpr int W = FOUR ? 4 : 1;
     for (int r = blockIdx.y; r < rows; r += gridDim.y) {
         const T* ar = a + r * a_stride;
@@ -252,30 +252,39 @@ __global__ void sigmoid_gate_kernel(const T* __restrict__ a, long long a_stride,
         T* o = out + r * out_stride;
         for (int c = (blockIdx.x * blockDim.x + threadIdx.x) * W; c < cols; c += gridDim.x * blockDim.x * W) {
             if (FOUR) {
-                const Four<T> av = *reinterpret_cast<const Four<T>*>(ar + c), gv = *reinterpret_cast<const Four<T>*>(gr + c);
-                Four<T> ov;
+                const Four<T> av = *reinterpret_cast<const Four<T>*>(ar + c);
+                Four<T> gv, ov;
+                // `per` > 1: one gate for every `per` consecutive columns (a number a head)
+                if (per > 1) {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) gv.v[u] = gr[(c + u) / per];
+                } else {
+                    gv = *reinterpret_cast<const Four<T>*>(gr + c);
+                }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) ov.v[u] = from_float<T>(to_float(av.v[u]) / (1.f + expf(-to_float(gv.v[u]))));
                 *reinterpret_cast<Four<T>*>(o + c) = ov;
             } else {
-                o[c] = from_float<T>(to_float(ar[c]) / (1.f + expf(-to_float(gr[c]))));
+                o[c] = from_float<T>(to_float(ar[c]) / (1.f + expf(-to_float(gr[c / per]))));
             }
         }
     }
 }
 
 WLLM_API int wllm_sigmoid_gate(const void* a, long long a_stride, const void* gate, long long gate_stride, void* out,
-                               long long out_stride, int is_bf16, int rows, int cols, hipStream_t stream) {
+                               long long out_stride, int is_bf16, int rows, int cols, int per, hipStream_t stream) {
     if (rows <= 0 || cols <= 0) return 0;
+    if (per < 1) return -1;
     const size_t four_bytes = 4 * (is_bf16 ? 2 : 4);
-    const bool four = cols % 4 == 0 && a_stride % 4 == 0 && gate_stride % 4 == 0 && out_stride % 4 == 0 &&
-                      reinterpret_cast<uintptr_t>(a) % four_bytes == 0 && reinterpret_cast<uintptr_t>(gate) % four_bytes == 0 &&
+    const bool gate_four = per > 1 || (gate_stride % 4 == 0 && reinterpret_cast<uintptr_t>(gate) % four_bytes == 0);
+    const bool four = cols % 4 == 0 && a_stride % 4 == 0 && gate_four && out_stride % 4 == 0 &&
+                      reinterpret_cast<uintptr_t>(a) % four_bytes == 0 &&
                       reinterpret_cast<uintptr_t>(out) % four_bytes == 0;
     const int per_row = four ? cols / 4 : cols;
     const dim3 grid(per_row < 4096 ? (per_row + 255) / 256 : 16, rows < 16384 ? rows : 16384);
 #define LAUNCH(T, FOUR)                                                                                              \
     sigmoid_gate_kernel<T, FOUR><<<grid, 256, 0, stream>>>(static_cast<const T*>(a), a_stride, static_cast<const T*>(gate), \
-                                                           gate_stride, static_cast<T*>(out), out_stride, rows, cols)
+                                                           gate_stride, static_cast<T*>(out), out_stride, rows, cols, per)
     if (is_bf16) {
         if (four) LAUNCH(bf16, true); else LAUNCH(bf16, false);
     } else {

@@ -113,6 +113,19 @@ MAX_HEADS = 1 << 16     # an item packs the key/value head and the tile's number
 MAX_TILES = 1 << 15     # tiles of 16 rows a segment may have for one key/value head (the item's int32 stays positive)
 
 
+
+def lowest_keys(pos: np.ndarray, window: int) -> np.ndarray:
+    """The lowest key the queries at positions `pos` see, from the one integer that names a mask (the
+    kernels' `lowest_key`): 0, every key; w > 0, a sliding window of w keys; -c < 0, chunks of c
+    positions counted from 0."""
+    pos = np.asarray(pos, dtype=np.int64)
+    if window > 0:
+        return np.maximum(0, pos - window + 1)
+    if window < 0:
+        return pos - pos % (-window)
+    return np.zeros_like(pos)
+
+
 def build_tile_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int):
     """Every segment, whatever its length, as tiles of 16 rows with their keys in chunks of `KEY_CHUNK`
     counted from key 0 (the float32 kernel takes nothing else): a tile's chunks are those its rows can
@@ -130,7 +143,7 @@ def build_tile_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
     row0 = tile * ROWS_PER_TILE
     first_pos = (ctx_len - q_len)[seg_of]
     last_row = np.minimum(rows[seg_of] - 1, row0 + ROWS_PER_TILE - 1)
-    lo = np.maximum(0, first_pos + row0 // group - window + 1) if window > 0 else np.zeros_like(row0)
+    lo = lowest_keys(first_pos + row0 // group, window)
     hi = first_pos + last_row // group + 1
     c0 = lo // KEY_CHUNK
     ns = (hi - 1) // KEY_CHUNK - c0 + 1
@@ -208,7 +221,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
     idx = np.nonzero(short)[0]
     if idx.size:
         first_pos = ctx_len[idx] - q_len[idx]
-        lo = np.maximum(0, first_pos - window + 1) if window > 0 else np.zeros_like(first_pos)
+        lo = lowest_keys(first_pos, window)
         c0 = lo // KEY_CHUNK
         c1 = (ctx_len[idx] - 1) // KEY_CHUNK
         ns = c1 - c0 + 1
@@ -263,7 +276,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         rb = (np.arange(int(n_blocks.sum())) - np.repeat(np.cumsum(n_blocks) - n_blocks, n_blocks)) * prefill_rows
         first_pos = (ctx_len - q_len)[seg_of]
         hi = first_pos + np.minimum(rows[seg_of] - 1, rb + prefill_rows - 1) // group + 1
-        lo = np.maximum(0, first_pos + rb // group - window + 1) if window > 0 else np.zeros_like(rb)
+        lo = lowest_keys(first_pos + rb // group, window)
         # a block's keys are cut into equal pieces whose boundaries are multiples of 32 counted from the block's
         # first group of 32
         lo32 = lo // 32 * 32

@@ -42,7 +42,7 @@ _SIGNATURES = {
     "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                     c_float, c_int, c_int, c_float, c_void_p],
+                                     c_float, c_int, c_int, c_float, c_void_p, c_void_p],
     "wllm_paged_attention_generic_chunk_keys": [],
     "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
@@ -183,6 +183,7 @@ class HipBackend:
 
     def plan_paged_attention(self, host_q_len, host_ctx_len, num_heads, num_kv_heads, head_dim, page_size, window,
                              dtype, device):
+        # `window`: w > 0 a sliding window, 0 none, -c < 0 chunks of c positions (the kernels' own convention)
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
         group, slots_of_device = num_heads // num_kv_heads, self._workgroup_slots(device)
@@ -234,8 +235,13 @@ class HipBackend:
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
-                        plan=None, softcap=0.0, exact_weights=False):
-        self._on_gpu(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out)
+                        plan=None, softcap=0.0, exact_weights=False, chunk=0, sinks=None):
+        self._on_gpu(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out, sinks)
+        if chunk:
+            # the kernels take one integer for the mask: w > 0 a sliding window, -c < 0 chunks of c positions
+            window = -int(chunk)
+        if sinks is not None and plan is not None:
+            raise KernelError("paged_attention: the matrix-core kernels have no sinks; give no plan")
         q_stride = qkv.shape[1]         # a row begins with the query heads; this many elements lie between two rows
         if plan is not None:
             if not self.mfma_attention_takes(qkv.dtype, head_dim, page_size):
@@ -294,7 +300,8 @@ class HipBackend:
             _ptr(qkv), _ptr(cache), int(qkv.dtype == torch.bfloat16), _ptr(block_tables), _ptr(token_segment),
             _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(self._generic_partial_o),
             _ptr(partial_ml), partial_tokens, max_ctx_len, qkv.shape[0], num_heads, num_kv_heads,
-            head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, self._stream()), "paged_attention")
+            head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, _ptr(sinks), self._stream()),
+            "paged_attention")
 
     @staticmethod
     def skinny_split(n: int, k: int) -> int:

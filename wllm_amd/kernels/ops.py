@@ -304,13 +304,16 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
                     seg_ctx_len: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                     head_dim: int, page_size: int, scale: float, window: int = 0,
                     max_q_len: int = 0, max_ctx_len: int = 0, plan=None, softcap: float = 0.0,
-                    exact_weights: bool = False) -> None:
+                    exact_weights: bool = False, chunk: int = 0, sinks: Optional[torch.Tensor] = None) -> None:
     """Softmax attention of every query over the keys of its own request in the paged cache.
 
     The batch is a row of segments; segment s holds tokens seg_q_start[s] .. +seg_q_len[s],
     the last seg_q_len[s] positions of a request that is seg_ctx_len[s] long after this
     step.  Token i of it is at position p = ctx_len - q_len + i and sees keys
-    max(0, p - window + 1) .. p (window 0: from key 0).  Query head h uses key/value head
+    max(0, p - window + 1) .. p (window 0: from key 0); with `chunk` c > 0 instead, the keys of its
+    own chunk of c positions counted from 0, (p // c) * c .. p.  With `sinks` (float32 [num_heads]) the
+    softmax's denominator holds exp(sinks[h]) once more: a term with no key and no value, not scaled
+    (only the kernels that run without a plan have it).  Query head h uses key/value head
     h // (num_heads // num_kv_heads).  Scores are scaled by `scale` and then, with `softcap` c > 0,
     bent to c * tanh(score / c); scores, softmax and the weighted sum accumulate in float32.
     The bfloat16 matrix-core kernels round a softmax weight to bfloat16 before they multiply it with the
@@ -341,12 +344,18 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
         _dense(t, name, torch.int32, (s,))
     _dense(out, "out", qkv.dtype, (n, num_heads * head_dim))
     _need(window >= 0, "window must not be negative")
+    _need(chunk >= 0 and not (chunk and window), "chunk must not be negative, and excludes a window")
+    if sinks is not None:
+        _dense(sinks, "sinks", torch.float32, (num_heads,))
+        _need(plan is None, "sinks: only the kernels that run without a plan have them")
     if n:
         backend().paged_attention(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len,
                                   out, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
                                   int(max_q_len), int(max_ctx_len), plan,
                                   **({"softcap": float(softcap)} if softcap else {}),
-                                  **({"exact_weights": True} if exact_weights else {}))
+                                  **({"exact_weights": True} if exact_weights else {}),
+                                  **({"chunk": int(chunk)} if chunk else {}),
+                                  **({"sinks": sinks} if sinks is not None else {}))
 
 
 def head_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
@@ -406,15 +415,22 @@ def _band(t: torch.Tensor, name: str, dtype, rows: int, cols: int) -> None:
           lambda: f"{name}: strides {t.stride()}: rows must be runs of consecutive elements")
 
 
-def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> None:
-    """out = a * sigmoid(gate), in float32, cast to T.  All T [n, c]; each may be a band of columns
-    of a wider tensor (a view whose rows are runs of consecutive elements); out may be a."""
+def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, per: int = 1) -> None:
+    """out = a * sigmoid(gate), in float32, cast to T.  a and out T [n, c]; gate T [n, c / per]: one
+    gate for every `per` consecutive columns (per = the head size: a number a head).  Each operand may
+    be a band of columns of a wider tensor (a view whose rows are runs of consecutive elements); out
+    may be a."""
     _need(a.dim() == 2 and a.dtype in _ACT, "a: expected T [n, c]")
     n, c = a.shape
-    for t, name in ((a, "a"), (gate, "gate"), (out, "out")):
+    _need(per >= 1 and c % per == 0, "per: a positive divisor of the columns")
+    for t, name in ((a, "a"), (out, "out")):
         _band(t, name, a.dtype, n, c)
+    _band(gate, "gate", a.dtype, n, c // per)
     if n and c:
-        call("sigmoid_gate", a, gate, out)
+        if per > 1:
+            call("sigmoid_gate", a, gate, out, per)
+        else:
+            call("sigmoid_gate", a, gate, out)
 
 
 def copy_columns(src: torch.Tensor, out: torch.Tensor) -> None:
@@ -675,6 +691,188 @@ def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
                               truncations)
 
 
+
+# ---- norms around the residual stream, general form ---------------------------------------------------
+NORM_KINDS = {"none": 0, "rms": 1, "layer": 2}
+
+
+class NormRecipe:
+    """A norm as the kernels take it: `kind` "rms" (v / sqrt(mean(v^2) + eps)) or "layer" ((v - mean) /
+    sqrt(mean((v - mean)^2) + eps), no bias), times (offset + weight); weight float32 [H]."""
+
+    def __init__(self, kind: str, weight: torch.Tensor, eps: float, offset: float = 0.0):
+        _need(kind in ("rms", "layer"), lambda: f"norm kind {kind!r}: expected rms or layer")
+        _dense(weight, "weight", torch.float32)
+        _need(weight.dim() == 1, "weight: expected one axis")
+        self.kind, self.weight, self.eps, self.offset = kind, weight, float(eps), float(offset)
+
+
+def norm_add(x: torch.Tensor, *, delta: Optional[torch.Tensor] = None, delta_norm: Optional[NormRecipe] = None,
+             out: Optional[torch.Tensor] = None, out_norm: Optional[NormRecipe] = None,
+             rows: Optional[torch.Tensor] = None) -> None:
+    """x += delta_norm(delta); out = out_norm(x), all in float32.
+
+    x float32 [n, H], the residual stream.  delta T [n, H] or a stack float32 [S, n, H] of partial sums
+    added in order; with `delta_norm` it is normalised before it is added (a norm behind a sublayer).
+    out T or float32 [m, H] (optional): the new x under `out_norm` (None: as it is, cast).  Without
+    `rows`, m = n and the sum is written back to x.  With `rows` (int32 [m]) only those rows are read,
+    x is left alone and out[i] belongs to row rows[i]."""
+    _dense(x, "x", torch.float32)
+    _need(x.dim() == 2, "x: expected [tokens, hidden]")
+    n, h = x.shape
+    _need(h <= 16384, "hidden: at most 16384")
+    if delta is not None:
+        if delta.dim() == 3:
+            _dense(delta, "delta", torch.float32, (delta.shape[0], n, h))
+            _need(delta.shape[0] >= 1, "delta: an empty stack")
+        else:
+            _dense(delta, "delta", _ACT, (n, h))
+    else:
+        _need(delta_norm is None, "delta_norm without delta")
+    for recipe, name in ((delta_norm, "delta_norm"), (out_norm, "out_norm")):
+        if recipe is not None:
+            _need(tuple(recipe.weight.shape) == (h,), lambda: f"{name}: weight of {tuple(recipe.weight.shape)}, expected [{h}]")
+    m = n
+    if rows is not None:
+        _dense(rows, "rows", torch.int32)
+        _need(rows.dim() == 1, "rows: expected one axis")
+        _need(out is not None, "rows without out")
+        m = rows.shape[0]
+    if out is not None:
+        _dense(out, "out", _ACT, (m, h))
+    else:
+        _need(out_norm is None, "out_norm without out")
+    if m and (delta is not None or out is not None):
+        call("norm_add", x, delta, delta_norm, out, out_norm, rows)
+
+
+def band_norm(bands: list, eps: float) -> None:
+    """RMS norm with a weight over bands of columns: for each (src, weight, count, out) of `bands` (one
+    or two), out[r] = src[r] / sqrt(sum(src[r]^2) / count + eps) * weight.  src T [n, c] and out T
+    [n, c'] with c' >= c may be bands of wider tensors and may be the same band; columns of out beyond c
+    become zero.  weight float32 [c].  `count` is the number of elements the mean is taken over (less
+    than c where the band carries padding that is always zero)."""
+    _need(1 <= len(bands) <= 2, "bands: one or two")
+    n, dtype = bands[0][0].shape[0], bands[0][0].dtype
+    _need(dtype in _ACT, "src: expected T")
+    for src, weight, count, out in bands:
+        _need(src.dim() == 2 and out.dim() == 2 and out.shape[1] >= src.shape[1], "out: at least as wide as src")
+        _band(src, "src", dtype, n, src.shape[1])
+        _band(out, "out", dtype, n, out.shape[1])
+        _dense(weight, "weight", torch.float32, (src.shape[1],))
+        _need(0 < count <= src.shape[1], "count: from 1 to the band's width")
+    if n:
+        call("band_norm", bands, float(eps))
+
+
+def gated_lookup(gate: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int, out: torch.Tensor,
+                 activation: str) -> None:
+    """out[r, c] = act(gate[r, c]) * table[ids[r], col0 + c].  gate, out T [n, d]; ids int32 [n];
+    table T [V, D] with col0 + d <= D."""
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
+    _dense(gate, "gate", _ACT)
+    _need(gate.dim() == 2, "gate: expected [n, d]")
+    n, d = gate.shape
+    _dense(ids, "ids", torch.int32, (n,))
+    _dense(table, "table", gate.dtype)
+    _need(table.dim() == 2 and 0 <= col0 and col0 + d <= table.shape[1], "table: expected [V, at least col0 + d]")
+    _dense(out, "out", gate.dtype, (n, d))
+    if n and d:
+        call("gated_lookup", gate, ids, table, int(col0), out, activation)
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor) -> None:
+    """A product head by head: y[r, h*O + o] = sum_k x[r, h*K + k] * w[h, o, k], float32 sums in ascending
+    order of k.  x T [n, heads*K] and y T [n, heads*O] may be bands of wider tensors; w T [heads, O, K]."""
+    _dense(w, "w", _ACT)
+    _need(w.dim() == 3, "w: expected [heads, out, in]")
+    heads, o, k = w.shape
+    _need(x.dim() == 2 and y.dim() == 2, "x, y: expected two axes")
+    n = x.shape[0]
+    _band(x, "x", w.dtype, n, heads * k)
+    _band(y, "y", w.dtype, n, heads * o)
+    if n:
+        call("head_linear", x, w, y)
+
+
+def causal_conv(inp: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, carried_offset: int,
+                token_segment: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
+                state_slots: torch.Tensor, out: torch.Tensor) -> None:
+    """A short causal convolution per channel over each segment, with silu, and the inputs it carries
+    from step to step.  inp T [n, C] (may be a band of a wider row); weight float32 [C, taps], the last
+    column the current token's; bias float32 [C]; out T [n, C] = silu(bias + sum_k weight[:, k] *
+    inp[t - (taps-1) + k]), where inputs before a segment's first token are the request's carried
+    rows: state float32 [slots, W] holds, from column `carried_offset` of row state_slots[segment],
+    [taps-1, C], the oldest first (zeros for a fresh request).  Afterwards the carried rows are the
+    segment's last taps-1 inputs (older carried rows move up where the segment is shorter)."""
+    _need(inp.dim() == 2 and inp.dtype in _ACT, "inp: expected T [n, C]")
+    n, c = inp.shape
+    _band(inp, "inp", inp.dtype, n, c)
+    _dense(weight, "weight", torch.float32)
+    _need(weight.dim() == 2 and weight.shape[0] == c and 1 <= weight.shape[1] <= 64, "weight: expected [C, taps]")
+    taps = weight.shape[1]
+    _dense(bias, "bias", torch.float32, (c,))
+    _dense(state, "state", torch.float32)
+    _need(state.dim() == 2 and 0 <= carried_offset and carried_offset + (taps - 1) * c <= state.shape[1],
+          "state: expected [slots, at least carried_offset + (taps-1)*C]")
+    _dense(token_segment, "token_segment", torch.int32, (n,))
+    s = seg_q_start.shape[0]
+    for t, name in ((seg_q_start, "seg_q_start"), (seg_q_len, "seg_q_len"), (state_slots, "state_slots")):
+        _dense(t, name, torch.int32, (s,))
+    _dense(out, "out", inp.dtype, (n, c))
+    if n:
+        call("causal_conv", inp, weight, bias, state, int(carried_offset), token_segment, seg_q_start, seg_q_len,
+             state_slots, out)
+
+
+def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+             state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
+             y: torch.Tensor, *, heads: int, groups: int, state_size: int, head_dim: int) -> None:
+    """The selective state-space recurrence over each segment's tokens in order, from and into the
+    request's carried state.  Per head h (group h // (heads // groups)) and token:
+        step = softplus(dt + dt_bias[h]);  S = exp(-exp(a_log[h]) * step) * S + step * B x^T;
+        y = S^T C + d_skip[h] * x
+    xbc T [n, heads*P + 2*groups*N]: x, then B, then C; dt T [n, heads] (may be a band of a wider row);
+    dt_bias, a_log, d_skip float32 [heads]; state float32 [slots, W], whose row state_slots[segment]
+    begins with S as [heads, N, P]; y float32 [n, heads*P].  All of the recurrence is float32."""
+    _dense(xbc, "xbc", _ACT)
+    inner = heads * head_dim
+    _need(heads > 0 and groups > 0 and heads % groups == 0, "heads must be a multiple of groups")
+    _need(0 < state_size <= 256, "state_size: from 1 to 256")
+    _need(xbc.dim() == 2 and xbc.shape[1] == inner + 2 * groups * state_size,
+          lambda: f"xbc: shape {tuple(xbc.shape)}, expected [n, {inner + 2 * groups * state_size}]")
+    n = xbc.shape[0]
+    _band(dt, "dt", xbc.dtype, n, heads)
+    for t, name in ((dt_bias, "dt_bias"), (a_log, "a_log"), (d_skip, "d_skip")):
+        _dense(t, name, torch.float32, (heads,))
+    _dense(state, "state", torch.float32)
+    _need(state.dim() == 2 and state.shape[1] >= heads * state_size * head_dim, "state: a row holds at least [heads, N, P]")
+    s = seg_q_start.shape[0]
+    for t, name in ((seg_q_start, "seg_q_start"), (seg_q_len, "seg_q_len"), (state_slots, "state_slots")):
+        _dense(t, name, torch.int32, (s,))
+    _dense(y, "y", torch.float32, (n, inner))
+    if n:
+        call("ssm_scan", xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y, heads, groups,
+             state_size, head_dim)
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, groups: int,
+                     eps: float) -> None:
+    """out = v / sqrt(mean over the part (v^2) + eps) * weight with v = y * silu(z), the row cut into
+    `groups` equal parts that are each divided by their own root mean square.  y float32 [n, W]; z T
+    [n, W] (may be a band of a wider row); weight float32 [W]; out T [n, W]."""
+    _dense(y, "y", torch.float32)
+    _need(y.dim() == 2, "y: expected [n, W]")
+    n, w = y.shape
+    _need(groups > 0 and w % groups == 0, "groups must divide the width")
+    _need(z.dtype in _ACT, "z: expected T")
+    _band(z, "z", z.dtype, n, w)
+    _dense(weight, "weight", torch.float32, (w,))
+    _dense(out, "out", z.dtype, (n, w))
+    if n:
+        call("gated_group_norm", y, z, weight, out, int(groups), float(eps))
+
+
 # ---- the framework's own operations that go through the same door as a part's ------------------
 def _register_own() -> None:
     from ctypes import c_float, c_int, c_longlong, c_void_p
@@ -709,10 +907,11 @@ def _register_own() -> None:
                           c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
                 launch=prepare)
     register_op("sigmoid_gate", entry_point="wllm_sigmoid_gate",
-                argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_void_p],
-                launch=lambda fn, stream, a, gate, out: fn(
+                argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_int,
+                          c_void_p],
+                launch=lambda fn, stream, a, gate, out, per=1: fn(
                     p(a), a.stride(0), p(gate), gate.stride(0), p(out), out.stride(0), int(a.dtype == torch.bfloat16),
-                    a.shape[0], a.shape[1], stream))
+                    a.shape[0], a.shape[1], per, stream))
     register_op("copy_columns", entry_point="wllm_copy_columns",
                 argtypes=[c_void_p, c_longlong, c_void_p, c_longlong, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, src, out: fn(
@@ -729,6 +928,68 @@ def _register_own() -> None:
     register_op("stream_add", entry_point="wllm_stream_add",
                 argtypes=[c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_int, c_int, c_void_p],
                 launch=add)
+
+
+    def norm_add_launch(fn, stream, x, delta, delta_norm, out, out_norm, rows):
+        splits, stride = 1, 0
+        if delta is not None and delta.dim() == 3:
+            splits, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+
+        def recipe(r):
+            return (NORM_KINDS[r.kind], p(r.weight), r.eps, r.offset) if r is not None else (0, p(None), 0.0, 0.0)
+
+        return fn(p(x), p(delta), int(delta is not None and delta.dtype == torch.bfloat16), splits, stride,
+                  *recipe(delta_norm), p(rows), p(out), int(out is not None and out.dtype == torch.bfloat16),
+                  *recipe(out_norm), out.shape[0] if out is not None else x.shape[0], x.shape[1], stream)
+
+    register_op("norm_add", entry_point="wllm_norm_add",
+                argtypes=[c_void_p, c_void_p, c_int, c_int, c_longlong, c_int, c_void_p, c_float, c_float, c_void_p, c_void_p,
+                          c_int, c_int, c_void_p, c_float, c_float, c_int, c_int, c_void_p],
+                launch=norm_add_launch)
+
+    def band_norm_launch(fn, stream, bands, eps):
+        args = []
+        for src, weight, count, out in bands:
+            args += [p(src), src.stride(0), src.shape[1], p(weight), float(count), p(out), out.stride(0), out.shape[1]]
+        if len(bands) == 1:
+            args += [p(None), 0, 0, p(None), 1.0, p(None), 0, 0]
+        first = bands[0][0]
+        return fn(*args, eps, int(first.dtype == torch.bfloat16), first.shape[0], stream)
+
+    one_band = [c_void_p, c_longlong, c_int, c_void_p, c_float, c_void_p, c_longlong, c_int]
+    register_op("band_norm", entry_point="wllm_band_norm", argtypes=one_band + one_band + [c_float, c_int, c_int, c_void_p],
+                launch=band_norm_launch)
+    register_op("gated_lookup", entry_point="wllm_gated_lookup",
+                argtypes=[c_void_p, c_void_p, c_void_p, c_longlong, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, gate, ids, table, col0, out, activation: fn(
+                    p(gate), p(ids), p(table), table.shape[1], col0, p(out), int(gate.dtype == torch.bfloat16),
+                    ACTIVATIONS[activation], gate.shape[0], gate.shape[1], stream))
+    register_op("head_linear", entry_point="wllm_head_linear",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, x, w, y: fn(
+                    p(x), x.stride(0), p(w), p(y), y.stride(0), int(w.dtype == torch.bfloat16), x.shape[0], w.shape[0],
+                    w.shape[1], w.shape[2], stream))
+    register_op("causal_conv", entry_point="wllm_causal_conv",
+                argtypes=[c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_longlong, c_longlong, c_void_p, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, inp, weight, bias, state, carried_offset, token_segment, seg_q_start, seg_q_len,
+                state_slots, out: fn(
+                    p(inp), inp.stride(0), p(weight), p(bias), p(state), state.stride(0), carried_offset, p(token_segment),
+                    p(seg_q_start), p(seg_q_len), p(state_slots), p(out), int(inp.dtype == torch.bfloat16), inp.shape[0],
+                    seg_q_start.shape[0], inp.shape[1], weight.shape[1], stream))
+    register_op("ssm_scan", entry_point="wllm_ssm_scan",
+                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y,
+                heads, groups, state_size, head_dim: fn(
+                    p(xbc), p(dt), dt.stride(0), p(dt_bias), p(a_log), p(d_skip), p(state), state.stride(0), p(seg_q_start),
+                    p(seg_q_len), p(state_slots), p(y), int(xbc.dtype == torch.bfloat16), seg_q_start.shape[0], heads, groups,
+                    state_size, head_dim, stream))
+    register_op("gated_group_norm", entry_point="wllm_gated_group_norm",
+                argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                launch=lambda fn, stream, y, z, weight, out, groups, eps: fn(
+                    p(y), p(z), z.stride(0), p(weight), p(out), int(z.dtype == torch.bfloat16), y.shape[0], y.shape[1],
+                    groups, eps, stream))
 
 
 _register_own()

@@ -1,4 +1,5 @@
-from wllm_amd.parts import attention, blocks, feed_forward, norms, positions  # noqa: F401  (register the kinds)
+from wllm_amd.parts import (attention, blocks, feed_forward, latent_attention, norms, positions,  # noqa: F401
+                            state_space)                                                     # (register the kinds)
 from wllm_amd.parts.model import (CausalLM, build_model, load_model, resolve_dtype, write_random_model_folder,
                                    write_random_model_from_config_json)
 from wllm_amd.parts.registry import (

@@ -15,6 +15,11 @@ rotation of interleaved pairs or of a part of the head, a unit norm of queries a
 that are the keys as projected (the row has no value heads), a cap on the scores, and an output
 gate whose projection is stacked behind the heads (row: queries, keys, [values], [gate]) and
 multiplied into the attention's result before the output projection, which may have a bias.
+Further options: value heads of another size than the key heads (both are padded to the larger in
+the row and in the cache, with zeros that add nothing to a score or a result); a mask of chunks
+instead of a window; an RMS norm with a weight over the whole query projection and over the whole key
+projection (`ops.band_norm`) in place of the norm of each head; a gate of one number a head; and a
+layer without key and value projections that reads another layer's cache with its own queries.
 """
 from __future__ import annotations
 
@@ -40,7 +45,18 @@ class PagedAttention:
         if spec.window is not None and spec.window <= 0:
             raise ValueError(f"window must be positive or None, got {spec.window}")
         plain = not (spec.softcap or spec.qk_norm_eps is not None or spec.values_are_keys or spec.gate_weight
-                     or spec.position.pairing == "interleaved")
+                     or spec.position.pairing == "interleaved" or spec.value_dim not in (None, spec.head_dim)
+                     or spec.chunk or spec.q_norm_weight or spec.k_norm_weight or not spec.owns_cache)
+        if spec.chunk is not None and (spec.chunk <= 0 or spec.window is not None):
+            raise ValueError(f"chunk must be positive and excludes a window, got chunk {spec.chunk}, window {spec.window}")
+        if (spec.q_norm_weight or spec.k_norm_weight) and spec.band_norm_eps is None:
+            raise ValueError("a norm over the whole query or key projection needs band_norm_eps")
+        if not spec.owns_cache and (spec.k_weight or spec.v_weight or spec.k_norm_weight or spec.values_are_keys
+                                    or spec.qk_norm_eps is not None or spec.position.kind != "none"):
+            raise ValueError("a layer without a cache of its own has no key or value projection, and its queries "
+                             "are neither rotated nor normed head by head")
+        if spec.gate_per_head and not spec.gate_weight:
+            raise ValueError("gate_per_head without a gate")
         if (plain and spec.head_dim % ops.HEAD_DIM_STEP) or not 0 < spec.head_dim <= ops.MAX_HEAD_DIM:
             raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of "
                              f"{ops.HEAD_DIM_STEP} up to {ops.MAX_HEAD_DIM}")
@@ -62,32 +78,47 @@ class PagedAttention:
         # rows of zeros in its projections (and columns of zeros in the output projection): the padding is zero
         # in queries, keys and values, adds nothing to a score or a result, and the unit norm divides by the
         # true size.  Only the general path does this.
-        self.dim = spec.head_dim if plain else -(-spec.head_dim // ops.HEAD_DIM_STEP) * ops.HEAD_DIM_STEP
+        self.vdim = spec.value_dim or spec.head_dim
+        largest = max(spec.head_dim, self.vdim)
+        self.dim = spec.head_dim if plain else -(-largest // ops.HEAD_DIM_STEP) * ops.HEAD_DIM_STEP
+        if not 0 < self.dim <= ops.MAX_HEAD_DIM:
+            raise ValueError(f"value_dim {self.vdim}: the attention kernels take heads up to {ops.MAX_HEAD_DIM}")
+        self.w_q_norm = self.w_k_norm = None
 
     @property
     def qkv_width(self) -> int:
         """Columns of the projected row: queries, keys, values (unless they are the keys), gate."""
         s = self.spec
-        heads = s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads + (s.num_heads if s.gate_weight else 0)
-        return heads * self.dim
+        return self.gate_offset + (self.gate_width if s.gate_weight else 0)
 
     @property
     def gate_offset(self) -> int:
         s = self.spec
-        return (s.num_heads + (1 if s.values_are_keys else 2) * s.num_kv_heads) * self.dim
+        kv = ((1 if s.values_are_keys else 2) * s.num_kv_heads) if s.owns_cache else 0
+        return (s.num_heads + kv) * self.dim
+
+    @property
+    def gate_width(self) -> int:
+        """Columns of the gate's projection: a number a head, or one for every element of the heads."""
+        return self.spec.num_heads if self.spec.gate_per_head else self.spec.num_heads * self.dim
 
     def expected_tensors(self) -> dict:
         s = self.spec
         q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
         out = {
             s.q_weight: ExpectedTensor((q, s.hidden_size)),
-            s.k_weight: ExpectedTensor((kv, s.hidden_size)),
-            s.o_weight: ExpectedTensor((s.hidden_size, q)),
+            s.o_weight: ExpectedTensor((s.hidden_size, s.num_heads * self.vdim)),
         }
-        if not s.values_are_keys:
-            out[s.v_weight] = ExpectedTensor((kv, s.hidden_size))
+        if s.owns_cache:
+            out[s.k_weight] = ExpectedTensor((kv, s.hidden_size))
+            if not s.values_are_keys:
+                out[s.v_weight] = ExpectedTensor((s.num_kv_heads * self.vdim, s.hidden_size))
         if s.gate_weight:
-            out[s.gate_weight] = ExpectedTensor((q, s.hidden_size))
+            out[s.gate_weight] = ExpectedTensor((s.num_heads if s.gate_per_head else s.num_heads * self.vdim, s.hidden_size))
+        if s.q_norm_weight:
+            out[s.q_norm_weight] = ExpectedTensor((q,), role="vector", init="norm")
+        if s.k_norm_weight and s.owns_cache:
+            out[s.k_norm_weight] = ExpectedTensor((kv,), role="vector", init="norm")
         for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv), (s.o_bias, s.hidden_size)):
             if name is not None:
                 out[name] = ExpectedTensor((width,), role="vector")
@@ -97,26 +128,39 @@ class PagedAttention:
 
     def load(self, fetch) -> None:
         s = self.spec
-        names = [s.q_weight, s.k_weight] + ([] if s.values_are_keys else [s.v_weight]) + ([s.gate_weight] if s.gate_weight else [])
-        pad = self.dim - s.head_dim
 
-        def heads_padded(t: torch.Tensor, axis: int) -> torch.Tensor:
-            """`t` with every head of `axis` (heads * head_dim long) followed by `pad` zeros."""
+        def heads_padded(t: torch.Tensor, axis: int, size: int = s.head_dim) -> torch.Tensor:
+            """`t` with every head of `axis` (heads * size long) followed by zeros up to the padded size."""
+            pad = self.dim - size
             if not pad:
                 return t
             shape = list(t.shape)
-            heads = shape[axis] // s.head_dim
-            t = t.unflatten(axis, (heads, s.head_dim))
+            heads = shape[axis] // size
+            t = t.unflatten(axis, (heads, size))
             zeros = torch.zeros(shape[:axis] + [heads, pad] + shape[axis + 1:], dtype=t.dtype, device=t.device)
             return torch.cat([t, zeros], dim=axis + 1).flatten(axis, axis + 1)
 
-        w = torch.cat([heads_padded(fetch.matrix(name), 0) for name in names], dim=0)
+        stacked = [heads_padded(fetch.matrix(s.q_weight), 0)]
+        if s.owns_cache:
+            stacked.append(heads_padded(fetch.matrix(s.k_weight), 0))
+            if not s.values_are_keys:
+                stacked.append(heads_padded(fetch.matrix(s.v_weight), 0, self.vdim))
+        if s.gate_weight:
+            gate = fetch.matrix(s.gate_weight)
+            stacked.append(gate if s.gate_per_head else heads_padded(gate, 0, self.vdim))
+        w = torch.cat(stacked, dim=0)
         self.w_qkv, self.t_qkv = load_matrix(fetch, w)        # the matrix and its tile-major copy
-        self.w_o, self.t_o = load_matrix(fetch, heads_padded(fetch.matrix(s.o_weight), 1))
+        self.w_o, self.t_o = load_matrix(fetch, heads_padded(fetch.matrix(s.o_weight), 1, self.vdim))
+        if s.q_norm_weight:
+            self.w_q_norm = fetch.to_device(heads_padded(fetch.vector(s.q_norm_weight), 0))
+        if s.k_norm_weight and s.owns_cache:
+            self.w_k_norm = fetch.to_device(heads_padded(fetch.vector(s.k_norm_weight), 0))
         if s.o_bias is not None:
             self.b_o = fetch.to_device(fetch.vector(s.o_bias))
         if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
             q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
+            if self.vdim != s.head_dim or not s.owns_cache:
+                raise NotImplementedError("biases of the projections beside value heads of another size")
             biases = [(s.q_bias, q), (s.k_bias, kv)] + ([] if s.values_are_keys else [(s.v_bias, kv)])
             # (the gate's projection, behind the heads in the row, has none: the bias is shorter than the row)
             found = [fetch.vector(name) if name is not None else None for name, _ in biases]
@@ -129,7 +173,8 @@ class PagedAttention:
         self.position.prepare(fetch.device)
 
     def cache_need(self) -> Optional[CacheNeed]:
-        return CacheNeed(self.spec.num_kv_heads, self.dim, self.spec.window)
+        s = self.spec
+        return CacheNeed(s.num_kv_heads, self.dim, s.window, s.release_chunk if s.chunk else None)
 
     def state_shape(self):
         return None
@@ -138,15 +183,17 @@ class PagedAttention:
         """Floating-point operations of `tokens` tokens whose queries see `keys` keys in all (what a
         measurement divides by its time)."""
         s = self.spec
-        return 2.0 * tokens * s.hidden_size * (self.qkv_width + s.num_heads * s.head_dim) + 4.0 * s.num_heads * s.head_dim * keys
+        return (2.0 * tokens * s.hidden_size * (self.qkv_width + s.num_heads * self.vdim)
+                + 2.0 * s.num_heads * (s.head_dim + self.vdim) * keys)
 
     def _work_items(self, ctx, page_size: int):
         """The step's work items for attention of this shape: made once a step, shared by all
         layers of the shape; of fixed shape and rewritten in place in a captured graph."""
         s = self.spec
         # (the plan depends on these alone: layers that differ in their rows' width or cap share it)
+        # (the mask as the one integer the plan takes: a window w > 0, chunks of c positions as -c)
         shape = dict(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=self.dim, page_size=page_size,
-                     window=s.window or 0)
+                     window=-s.chunk if s.chunk else (s.window or 0))
 
         def build(c):
             if c.captured:
@@ -174,7 +221,28 @@ class PagedAttention:
         inv_freq = self.position.inv_freq
         apply = getattr(self.position, "apply", None)
         rotary_dim = 2 * inv_freq.shape[0] if inv_freq is not None else s.head_dim
-        if not self.plain:
+        if not self.plain and (self.w_q_norm is not None or not s.owns_cache):
+            if apply is not None:
+                raise NotImplementedError("a position encoding with a step of its own beside the attention's options")
+            # the whole projections are normed before the heads are split: the sums of a split product are
+            # made here, and the norm kernel takes the query band and the key band in one launch
+            ops.linear(h, self.w_qkv, qkv, self.t_qkv)
+            q_width, kv_width = s.num_heads * self.dim, s.num_kv_heads * self.dim
+            bands = []
+            if self.w_q_norm is not None:
+                bands.append((qkv[:, :q_width], self.w_q_norm, s.num_heads * s.head_dim, qkv[:, :q_width]))
+            if self.w_k_norm is not None:
+                bands.append((qkv[:, q_width:q_width + kv_width], self.w_k_norm, s.num_kv_heads * s.head_dim,
+                              qkv[:, q_width:q_width + kv_width]))
+            if bands:
+                ops.band_norm(bands, s.band_norm_eps)
+            if s.owns_cache:
+                ops.head_prepare(
+                    qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage, num_heads=s.num_heads,
+                    num_kv_heads=s.num_kv_heads, head_dim=self.dim, page_size=pages.page_size,
+                    interleaved=getattr(self.position, "interleaved", False), norm_eps=s.qk_norm_eps,
+                    values_are_keys=s.values_are_keys, norm_dim=s.head_dim)
+        elif not self.plain:
             if apply is not None:
                 raise NotImplementedError("a position encoding with a step of its own beside the attention's options")
             projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
@@ -211,12 +279,13 @@ class PagedAttention:
             ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=self.dim,
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
-            plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0, exact_weights=s.weights_in_float32)
+            plan=self._work_items(ctx, pages.page_size), softcap=s.softcap or 0.0, exact_weights=s.weights_in_float32,
+            chunk=s.chunk or 0)
         if s.gate_weight:
             # the gate's columns lie behind the heads in the projected row
-            gate = qkv[:, self.gate_offset:self.gate_offset + s.num_heads * self.dim]
+            gate = qkv[:, self.gate_offset:self.gate_offset + self.gate_width]
             target = product_input if product_input is not None else attn
-            ops.sigmoid_gate(attn, gate, target)
+            ops.sigmoid_gate(attn, gate, target, per=self.dim if s.gate_per_head else 1)
             attn = target
         elif product_input is not None:
             ops.copy_columns(attn, product_input)

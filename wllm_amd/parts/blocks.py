@@ -13,6 +13,11 @@ projection), and the sum of two products is one product over the two inputs side
 [a | f] [Wo | Wd]^T.  The block lays the two weights side by side at load, lets the parts write
 their products' inputs into the two bands of one buffer, and makes that one product: the sum is
 formed in the product's float32 accumulators, and the stream sees one contribution.
+
+"sandwich": x += post(mixer(pre(x))); x += post(feed_forward(pre(x))): a norm behind each sublayer as
+well as before it, then, if the layer has one, a per-layer token input that reads the stream itself.
+A sublayer's product stays pending together with the norm it has to pass (`pending_norm`), and the
+next norm kernel normalises it, adds it and normalises the sum for the next sublayer in one pass.
 """
 from __future__ import annotations
 
@@ -40,10 +45,22 @@ class ResidualStream:
         self.x = x
         self.pending = pending
         self.pending_bias: Optional[torch.Tensor] = None      # float32 [H]: a row that comes with `pending`
+        self.pending_norm = None       # an `ops.NormRecipe`: `pending` passes this norm before it is added
         self.sumsq: Optional[torch.Tensor] = None      # float32 [n, bands]: sums of squares of x as it is now
 
     def normed(self, norm, out: torch.Tensor, rows=None) -> torch.Tensor:
         """norm(x + pending).  Without `rows` the sum becomes the new x."""
+        if self.pending_norm is not None:
+            if getattr(norm, "takes_delta_norm", False) and self.pending_bias is None:
+                norm.forward(self.x, out, delta=self.pending, rows=rows, delta_norm=self.pending_norm)
+                if rows is None:
+                    self.pending = self.pending_norm = None
+                    self.sumsq = None
+                return out
+            if rows is not None:
+                raise NotImplementedError("gathered rows of a stream whose pending part has a norm, under a norm "
+                                          "that cannot apply it")
+            self.settle()
         if self.pending_bias is not None:
             norm.forward(self.x, out, delta=self.pending, rows=rows, delta_bias=self.pending_bias)
         else:
@@ -57,6 +74,12 @@ class ResidualStream:
         """x takes what is pending, and `addend` (float32, x's shape) with it, without a norm."""
         if self.pending is None and self.pending_bias is None and addend is None:
             return
+        if self.pending_norm is not None:
+            ops.norm_add(self.x, delta=self.pending, delta_norm=self.pending_norm)
+            self.pending = self.pending_norm = None
+            self.sumsq = None
+            if self.pending_bias is None and addend is None:
+                return
         ops.stream_add(self.x, addend, self.pending, self.pending_bias)
         self.pending = self.pending_bias = None
         self.sumsq = None
@@ -70,9 +93,32 @@ class ResidualStream:
             return norm.on_load(self.x, self.sumsq, ctx.dtype)
         return self.normed(norm, ctx.buffer("normed", (n, hidden), ctx.dtype))
 
-    def add(self, ctx, y) -> None:
+    def as_activations(self, ctx) -> torch.Tensor:
+        """The stream itself (what is pending added) in the activation type, for a part that reads it
+        without a norm."""
+        n, hidden = self.x.shape
+        if ctx.dtype == torch.float32:
+            self.settle()
+            return self.x
+        out = ctx.buffer("stream_cast", (n, hidden), ctx.dtype)
+        if self.pending_bias is not None:
+            self.settle()
+        ops.norm_add(self.x, delta=self.pending, delta_norm=self.pending_norm, out=out)
+        self.pending = self.pending_norm = None
+        self.sumsq = None
+        return out
+
+    def add(self, ctx, y, norm=None) -> None:
+        """`norm` (a norm part): the contribution passes it before it is added (a norm behind a sublayer)."""
         if self.pending is not None or self.pending_bias is not None:
             raise RuntimeError("a contribution is already pending; normalise before adding another")
+        if norm is not None:
+            if isinstance(y, Product):
+                if y.bias is not None:
+                    raise NotImplementedError("a product with a bias under a norm behind its sublayer")
+                y = y.make(ctx)
+            self.pending, self.pending_norm = y, norm.recipe()
+            return
         if isinstance(y, Product):
             n, hidden = self.x.shape
             self.pending_bias = y.bias
@@ -154,3 +200,41 @@ class ParallelBlock:
         f = self.feed_forward.forward(ctx, h, product_input=both[:, self.k_mixer:])
         bias = a.bias if f.bias is None else (f.bias if a.bias is None else a.bias + f.bias)
         stream.add(ctx, Product("block_out", both, self.w_joint, self.t_joint, bias=bias))
+
+
+@register_block("sandwich")
+class SandwichBlock:
+    """x += post(mixer(pre(x))); x += post(feed_forward(pre(x))); then the layer's token input."""
+
+    def __init__(self, spec: BlockSpec):
+        if spec.mixer_post_norm is None or (spec.feed_forward is not None and (
+                spec.feed_forward_norm is None or spec.feed_forward_post_norm is None)):
+            raise ValueError("a sandwich block has a norm before and behind each of its sublayers")
+        self.spec = spec
+        self.mixer = build_mixer(spec.mixer)
+        self.mixer_norm = build_norm(spec.mixer_norm)
+        self.mixer_post_norm = build_norm(spec.mixer_post_norm)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_post_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = build_feed_forward(spec.feed_forward)
+            self.feed_forward_norm = build_norm(spec.feed_forward_norm)
+            self.feed_forward_post_norm = build_norm(spec.feed_forward_post_norm)
+        self.side = None
+        if spec.side is not None:
+            from wllm_amd.parts.token_side import TokenSide
+            self.side = TokenSide(spec.side)
+
+    def parts(self) -> list:
+        own = [self.mixer_norm, self.mixer, self.mixer_post_norm]
+        if self.feed_forward is not None:
+            own += [self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm]
+        return own + ([self.side] if self.side is not None else [])
+
+    def forward(self, ctx, entry: int, stream: ResidualStream) -> None:
+        h = stream.input_for(ctx, self.mixer_norm, self.mixer)
+        stream.add(ctx, self.mixer.forward(ctx, entry, h), norm=self.mixer_post_norm)
+        if self.feed_forward is not None:
+            h = stream.input_for(ctx, self.feed_forward_norm, self.feed_forward)
+            stream.add(ctx, self.feed_forward.forward(ctx, h), norm=self.feed_forward_post_norm)
+        if self.side is not None:
+            stream.add(ctx, self.side.forward(ctx, stream.as_activations(ctx)), norm=self.side.norm)
