@@ -89,7 +89,10 @@ class PagedAttention:
     def qkv_width(self) -> int:
         """Columns of the projected row: queries, keys, values (unless they are the keys), gate."""
         s = self.spec
-        return self.gate_offset + (self.gate_width if s.gate_weight else 0)
+        width = self.gate_offset + (self.gate_width if s.gate_weight else 0)
+        # a gate of a number a head can leave the row at any width; the kernels read rows that begin at
+        # multiples of 16 bytes, so the row is padded (with zero rows of the stacked weight)
+        return -(-width // 8) * 8 if s.gate_per_head else width
 
     @property
     def gate_offset(self) -> int:
@@ -149,6 +152,8 @@ class PagedAttention:
             gate = fetch.matrix(s.gate_weight)
             stacked.append(gate if s.gate_per_head else heads_padded(gate, 0, self.vdim))
         w = torch.cat(stacked, dim=0)
+        if w.shape[0] < self.qkv_width:
+            w = torch.cat([w, torch.zeros(self.qkv_width - w.shape[0], w.shape[1], dtype=w.dtype, device=w.device)], dim=0)
         self.w_qkv, self.t_qkv = load_matrix(fetch, w)        # the matrix and its tile-major copy
         self.w_o, self.t_o = load_matrix(fetch, heads_padded(fetch.matrix(s.o_weight), 1, self.vdim))
         if s.q_norm_weight:
