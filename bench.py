@@ -233,7 +233,8 @@ def run_compare(args) -> dict:
             for batch in (1, 8, 64):
                 k = max(8, args.steps // 2)
                 d, ctx_len = measure_decode(model, batch, args.context, k, 4, args.block_size, graphs)
-                gbs = (model.weight_bytes() + batch * ctx_len * kv_bytes_per_token(model)) / (d / k) / 1e9
+                state = 2 * model.state_bytes() if hasattr(model, "state_bytes") else 0     # read and written a step
+                gbs = (model.weight_bytes() + batch * (ctx_len * kv_bytes_per_token(model) + state)) / (d / k) / 1e9
                 points[f"{key}_decode_b{batch}"] = round(k * batch / d, 1)
                 points[f"{key}_decode_b{batch}_ms"] = round(1000.0 * d / k, 4)
                 points[f"{key}_decode_b{batch}_frac"] = round(gbs / PEAK_HBM_GBS, 4)
@@ -265,7 +266,7 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "stress", "compare"],
                     help="decode: the contract's line; stress: continuous batching of 64 mixed requests; compare: prefill "
                          "and decode of the pairs of shapes of --compare, one model after the other")
-    ap.add_argument("--compare", default="tasosun-2b:gemma-2b,tasosun-7b:gemma-7b",
+    ap.add_argument("--compare", default="tasosun-2b:gemma-2b,tasosun-7b:gemma-7b",   # also: tokuvik-2b:gemma-2b
                     help="compare: pairs of shapes (named, or config.json files), new:closest, with commas between pairs")
     ap.add_argument("--stress-requests", type=int, default=64)
     ap.add_argument("--row-multiple", type=int, default=256,

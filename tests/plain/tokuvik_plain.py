@@ -120,6 +120,31 @@ def causal_conv(u, weight, bias):
     return out
 
 
+def state_space_recurrence(x, b, c, dt, a_log, d_skip, state=None):
+    """x [t, heads, p]; b, c [t, groups, n]; dt [t, heads] (after softplus); a_log, d_skip [heads].
+    S_t = exp(-exp(a_log) dt_t) S_(t-1) + dt_t B_t x_t^T;  y_t = S_t^T C_t + d_skip x_t.  Returns y [t, heads, p]
+    and the last S [heads, n, p]; `state`: the S to start from (zeros if None)."""
+    t, heads, p = x.shape
+    per_group = heads // b.shape[1]
+    decay = torch.exp(-torch.exp(a_log) * dt)
+    s = torch.zeros(heads, b.shape[2], p, dtype=x.dtype) if state is None else state
+    ys = []
+    for i in range(t):
+        bi = b[i].repeat_interleave(per_group, dim=0)      # [heads, n]
+        ci = c[i].repeat_interleave(per_group, dim=0)
+        s = decay[i][:, None, None] * s + dt[i][:, None, None] * bi[:, :, None] * x[i][:, None, :]
+        ys.append(torch.einsum("hnp,hn->hp", s, ci) + d_skip[:, None] * x[i])
+    return torch.stack(ys), s
+
+
+def gated_group_norm(y, z, w, parts: int, eps):
+    """y * silu(z), each of `parts` equal parts of a row divided by its own root mean square, times w."""
+    t, width = y.shape
+    v = (y * silu(z)).view(t, parts, width // parts)
+    v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
+    return v.reshape(t, width) * w
+
+
 def mamba2_mixer(h, w, p, mixer, eps):
     t = h.shape[0]
     heads, vdim, n, groups = mixer["heads"], mixer["vdim"], mixer["state"], mixer["groups"]
@@ -131,20 +156,8 @@ def mamba2_mixer(h, w, p, mixer, eps):
     b = xbc[:, inner:inner + groups * n].view(t, groups, n)
     c = xbc[:, inner + groups * n:].view(t, groups, n)
     dt = softplus(dt + w[p + "dt_bias"])                   # [t, heads]
-    decay = torch.exp(-torch.exp(w[p + "A_log"]) * dt)     # [t, heads]
-    per_group = heads // groups
-    state = torch.zeros(heads, n, vdim, dtype=h.dtype)
-    ys = []
-    for i in range(t):
-        bi = b[i].repeat_interleave(per_group, dim=0)      # [heads, n]
-        ci = c[i].repeat_interleave(per_group, dim=0)
-        state = decay[i][:, None, None] * state + dt[i][:, None, None] * bi[:, :, None] * x[i][:, None, :]
-        ys.append(torch.einsum("hnp,hn->hp", state, ci) + w[p + "D"][:, None] * x[i])
-    y = torch.stack(ys).reshape(t, inner) * silu(z)
-    parts = mixer["norm_groups"]
-    y = y.view(t, parts, inner // parts)
-    y = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps)
-    y = y.reshape(t, inner) * w[p + "norm"]
+    y, _ = state_space_recurrence(x, b, c, dt, w[p + "A_log"], w[p + "D"])
+    y = gated_group_norm(y.reshape(t, inner), z, w[p + "norm"], mixer["norm_groups"], eps)
     return y @ w[p + "o"].T
 
 

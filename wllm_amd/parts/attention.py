@@ -188,6 +188,8 @@ class PagedAttention:
         """Floating-point operations of `tokens` tokens whose queries see `keys` keys in all (what a
         measurement divides by its time)."""
         s = self.spec
+        if s.chunk:
+            keys = min(keys, tokens * (s.chunk + 1) / 2.0)      # a query sees half a chunk on average
         return (2.0 * tokens * s.hidden_size * (self.qkv_width + s.num_heads * self.vdim)
                 + 2.0 * s.num_heads * (s.head_dim + self.vdim) * keys)
 

@@ -128,6 +128,14 @@ class CausalLM:
         self.embed_scale = scale
         self.dtype, self.device = dtype, device
 
+    def state_bytes(self) -> int:
+        """Bytes of fixed-size state one request carries over all layers (a decode step reads and writes them)."""
+        total = 0
+        for shape in self.state_shapes().values():
+            dims, size = (shape.shape, shape.dtype.itemsize) if hasattr(shape, "shape") else (shape, 4)
+            total += math.prod(dims) * size
+        return total
+
     def weight_bytes(self) -> int:
         """Bytes of every weight a step reads once (the tied table counts once)."""
         seen, total = set(), 0
@@ -136,7 +144,9 @@ class CausalLM:
         for block in self.blocks:
             for part in block.parts():
                 # a tile-major copy (t_*) holds the same numbers as its matrix; a step reads one of the two
-                tensors.extend(v for k, v in vars(part).items() if isinstance(v, torch.Tensor) and not k.startswith("t_"))
+                # (nor a table of which a step reads one row a token: the part names it in `lookup_tables`)
+                tensors.extend(v for k, v in vars(part).items() if isinstance(v, torch.Tensor) and not k.startswith("t_")
+                               and k not in getattr(part, "lookup_tables", ()))
         for t in tensors:
             if t is not None and t.data_ptr() not in seen:
                 seen.add(t.data_ptr())

@@ -19,6 +19,8 @@ from wllm_amd.weights.checkpoint import ExpectedTensor
 
 
 class TokenSide:
+    lookup_tables = ("table",)      # read a row a token, not whole: no part of the weights a step streams
+
     def __init__(self, spec: TokenSideSpec):
         if spec.activation not in ops.ACTIVATIONS:
             raise ValueError(f"activation {spec.activation!r} is not implemented; known: {ops.ACTIVATIONS}")
