@@ -27,9 +27,12 @@ LENGTHS = {"trio": [70, 45, 150, 33, 58], "odd": [40, 66, 25, 151], "sharp": [80
 FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions, "mixed": trace_mixed}
 # a row's distance from the plain implementation, as a share of the row's own size: float32 sums in another
 # order; bfloat16 activations through some ten roundings a layer
-RELATIVE = {torch.float32: 1e-4, torch.bfloat16: 6e-2}
-# the sharp model multiplies every rounding by some hundred (a lost key still moves a row by far more than this)
-SHARP_RELATIVE = {torch.float32: 6e-4, torch.bfloat16: 0.5}
+# (measured: float32 rows lie 1e-6 to 7e-6 away; bfloat16 rows 0.4 to 1% a handful of layers, with a row in a hundred up to
+# 8% where rounding decides between two keys)
+BOUND = {torch.float32: dict(relative=1e-4), torch.bfloat16: dict(relative=0.04, outliers=0.05, ceiling=6.0)}
+# the sharp model multiplies every rounding by some hundred (in float32 a lost key still moves a row by far more than
+# this; in bfloat16 single keys change places, and only the bulk of the rows says anything)
+SHARP_BOUND = {torch.float32: dict(relative=6e-4), torch.bfloat16: dict(relative=0.3, outliers=0.2, ceiling=10.0)}
 
 
 def close(got, ref, dtype, what="", scale=1.0):
@@ -299,7 +302,7 @@ def test_replay_matches_plain(folders, name, family, dtype):
         got = replay_and_collect(TraceReplayer(runner), trace)
     runner.cache.check()
     assert not runner.cache.requests
-    compare_rows(got, exact, relative=(SHARP_RELATIVE if name == "sharp" else RELATIVE)[dtype])
+    compare_rows(got, exact, **(SHARP_BOUND if name == "sharp" else BOUND)[dtype])
 
 
 @pytest.mark.parametrize("seed", range(10))
@@ -317,7 +320,7 @@ def test_configurations_drawn_at_random(tmp_path, seed):
             with torch.inference_mode():
                 got = replay_and_collect(TraceReplayer(runner), trace)
             runner.cache.check()
-            compare_rows(got, exact, relative=RELATIVE[dtype])
+            compare_rows(got, exact, **BOUND[dtype])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -337,7 +340,7 @@ def test_long_decoding_through_chunks_in_a_small_pool(folders, dtype):
         with torch.inference_mode():
             got = replay_and_collect(TraceReplayer(runner), trace_tail(requests, tail=260))
         runner.cache.check()
-    compare_rows(got, exact, relative=SHARP_RELATIVE[dtype])
+    compare_rows(got, exact, **SHARP_BOUND[dtype])
 
 
 def test_a_row_does_not_depend_on_the_batch_or_the_cut(folders):

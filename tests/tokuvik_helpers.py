@@ -188,16 +188,22 @@ def _centred_rms(d: torch.Tensor) -> float:
     return (d - d.mean()).pow(2).mean().sqrt().item()
 
 
-def compare_rows(collected: dict, exact: dict, *, relative: float) -> float:
+def compare_rows(collected: dict, exact: dict, *, relative: float, outliers: float = 0.0, ceiling: float = 1.0) -> float:
     """Every collected row against the plain implementation's: the root mean square of the difference,
-    its mean taken off, may be `relative` of the exact row's own.  Returns the worst error in units of
-    its bound and names the first row beyond it."""
-    worst = 0.0
+    its mean taken off, may be `relative` of the exact row's own.  bfloat16 rounding now and then decides
+    between two keys of almost equal score, and the row is then far off though nothing is wrong: a share
+    `outliers` of the rows may lie beyond the bound, up to `ceiling` times it.  Returns the worst error in
+    units of the bound and names the first row beyond what is allowed."""
+    errors = {}
     for (rid, pos) in sorted(collected, key=lambda k: (str(k[0]), k[1])):
         got, ref = collected[(rid, pos)].double(), exact[rid][pos].double()
         assert torch.isfinite(got).all(), f"request {rid!r} position {pos}: logits are not finite"
         bound = relative * max(_centred_rms(ref), 1e-3)
-        err = _centred_rms(got - ref) / bound
-        assert err <= 1.0, f"request {rid!r} position {pos}: {err:.2f} x the bound ({_centred_rms(got - ref):.3e} against {bound:.3e})"
-        worst = max(worst, err)
+        errors[(rid, pos)] = _centred_rms(got - ref) / bound
+    beyond = {k: e for k, e in errors.items() if e > 1.0}
+    worst = max(errors.values())
+    assert len(beyond) <= outliers * len(errors), (
+        f"{len(beyond)} of {len(errors)} rows beyond the bound; the first: request {next(iter(beyond))[0]!r} position "
+        f"{next(iter(beyond))[1]}: {next(iter(beyond.values())):.2f} x the bound")
+    assert worst <= max(ceiling, 1.0), f"a row is {worst:.2f} x the bound"
     return worst
