@@ -240,6 +240,8 @@ def _attention_problem(dtype, nh, nkv, d, ps, segs, seed, extra_columns):
     (6, 1, 28, 8, 19, True, [(1, 20), (1, 19), (40, 40), (3, 230)]),                        # ... with sinks
     (5, 1, 96, 16, 0, True, [(1, 300), (70, 70), (1, 1), (2, 131)]),                        # sinks, no mask, many heads on one
     (12, 1, 64, 16, 0, True, [(1, 129), (30, 45)]),
+    (20, 1, 256, 16, 0, True, [(1, 700), (300, 300), (64, 1000)]),                          # keys cut into pieces: the reduce kernels
+    (4, 2, 128, 8, 50, True, [(1, 49), (1, 50), (1, 51), (200, 230)]),
 ])
 def test_chunks_and_sinks_in_every_attention_kernel(dtype, nh, nkv, d, ps, chunk, sinks, segs):
     """Keys just inside and just outside a chunk's edge, decoded alone and inside prompts, with scores so
@@ -254,10 +256,9 @@ def test_chunks_and_sinks_in_every_attention_kernel(dtype, nh, nkv, d, ps, chunk
                   max_q_len=int(q_len.max()), max_ctx_len=int(ctx.max()), exact_weights=True)
     if sinks:
         kwargs["sinks"] = sink.to(DEV)
-    else:
-        kwargs["plan"] = ops.plan_paged_attention(q_len.numpy(), ctx.numpy(), num_heads=nh, num_kv_heads=nkv, head_dim=d,
-                                                  page_size=ps, window=-chunk, dtype=dtype, device=torch.device(DEV))
-        assert (kwargs["plan"] is not None) == (d % 32 == 0 and ps % 4 == 0)
+    kwargs["plan"] = ops.plan_paged_attention(q_len.numpy(), ctx.numpy(), num_heads=nh, num_kv_heads=nkv, head_dim=d,
+                                              page_size=ps, window=-chunk, dtype=dtype, device=torch.device(DEV))
+    assert (kwargs["plan"] is not None) == (d % 32 == 0 and ps % 4 == 0)
     ops.paged_attention(*args, **kwargs)
     torch.cuda.synchronize()
     kview = cache[:, 0].view(-1, nkv, ps, d).double()

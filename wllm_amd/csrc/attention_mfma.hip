@@ -65,7 +65,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                             const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                             float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                             int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
-                            int q_stride, float cap_scale, float softcap) {
+                            int q_stride, float cap_scale, float softcap, const float* __restrict__ sinks) {
     constexpr int DC = HD / 32;   // 32-wide chunks of the head for the score product
     constexpr int DT = HD / 16;   // 16-row tiles of out^T
     // Shared memory, a part for each wavefront, used four times: three workgroups share a compute
@@ -301,7 +301,10 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                 f_of[w] = exp2f((m_of[w] - m_use) * scale_log2e);       // 0 for a wavefront without keys
                 l_all = fmaf(l_of[w], f_of[w], l_all);
             }
-            inv = 1.f / l_all;
+            // a sink: exp(sink of the head) once more in the denominator of a row that is finished here
+            // (the maximum is held in the exponent's own units: times scale_log2e it is in powers of two)
+            const float sink_term = (sinks && partial_slot < 0) ? exp2f(sinks[head] * 1.4426950408889634f - m_use * scale_log2e) : 0.f;
+            inv = 1.f / (l_all + sink_term);
         }
         if (row_valid) {
 #pragma unroll
@@ -342,7 +345,7 @@ __global__ void __launch_bounds__(HD)
 attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
                         const float* __restrict__ partial_ml, const int* __restrict__ seg_q_start,
                         const int* __restrict__ seg_q_len, bf16* __restrict__ out, int num_heads, int num_kv_heads,
-                        float scale_log2e) {
+                        float scale_log2e, const float* __restrict__ sinks) {
     // one workgroup per (item, row); one thread per element of the head; the loads of the
     // splits do not depend on each other.  Reduce items are 8 int32: segment, key/value head, first
     // slot, number of splits, first row of the tile within the segment, slots between two splits.
@@ -388,6 +391,7 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
     }
     const int row = row0 + r;
     const int tok = row / group, head = kvh * group + row % group;
+    if (sinks) den += exp2f(sinks[head] * 1.4426950408889634f - m * scale_log2e);
     out[(static_cast<size_t>(q_start + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
 }
 
@@ -400,7 +404,7 @@ __global__ void __launch_bounds__(HD)
 attention_reduce_wide_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
                              const float* __restrict__ partial_ml, const int* __restrict__ seg_q_start,
                              const int* __restrict__ seg_q_len, bf16* __restrict__ out, int num_heads,
-                             int num_kv_heads, float scale_log2e) {
+                             int num_kv_heads, float scale_log2e, const float* __restrict__ sinks) {
     const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * kItemInts;
     const int seg = item[0], kvh = item[1], first = item[2], splits = item[3], row0 = item[4];
     if (seg < 0) return;
@@ -444,6 +448,7 @@ attention_reduce_wide_kernel(const int* __restrict__ reduce_items, const float* 
     }
     const int row = row0 + r;
     const int tok = row / group, head = kvh * group + row % group;
+    if (sinks) den += exp2f(sinks[head] * 1.4426950408889634f - m * scale_log2e);
     uint2 w;
     w.x = pack2_bf16(num[0] / den, num[1] / den);
     w.y = pack2_bf16(num[2] / den, num[3] / den);
@@ -473,6 +478,7 @@ struct AttentionArguments {
     int q_stride;
     float cap_scale, softcap;
     int split_weights;
+    const float* sinks;
     hipStream_t stream;
 };
 
@@ -481,7 +487,7 @@ int launch_items(const AttentionArguments& a) {
     paged_attention_mfma_kernel<HD, V16, SPLIT><<<a.num_items, 256, 0, a.stream>>>(
         a.qkv, a.cache, a.block_tables, a.items, a.live_items, a.seg_q_start, a.seg_q_len, a.seg_ctx_len, a.out,
         a.partial_o, a.partial_ml, a.num_heads, a.num_kv_heads, a.page_size, a.max_pages, a.scale_log2e, a.window,
-        a.q_stride, a.cap_scale, a.softcap);
+        a.q_stride, a.cap_scale, a.softcap, a.sinks);
     return 0;
 }
 
@@ -496,11 +502,11 @@ int launch_all(const AttentionArguments& a) {
     if (a.num_reduce_items >= 64) {
         attention_reduce_wide_kernel<HD><<<dim3(a.num_reduce_items, kRowsPerTile / 4), HD, 0, a.stream>>>(
             a.reduce_items, a.partial_o, a.partial_ml, a.seg_q_start, a.seg_q_len, a.out, a.num_heads, a.num_kv_heads,
-            a.scale_log2e);
+            a.scale_log2e, a.sinks);
     } else if (a.num_reduce_items > 0) {
         attention_reduce_kernel<HD><<<dim3(a.num_reduce_items, kRowsPerTile), HD, 0, a.stream>>>(
             a.reduce_items, a.partial_o, a.partial_ml, a.seg_q_start, a.seg_q_len, a.out, a.num_heads, a.num_kv_heads,
-            a.scale_log2e);
+            a.scale_log2e, a.sinks);
     }
     return launch_status();
 }
@@ -515,7 +521,7 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
                                        const int* seg_ctx_len, void* out, float* partial_o, float* partial_ml,
                                        int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
                                        float scale, int window, int q_stride, float softcap, int split_weights,
-                                       hipStream_t stream) {
+                                       const float* sinks, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         num_heads >= (1 << 16))       // an item holds a key/value head and a tile's first row in 16 bits each
         return -1;
@@ -527,7 +533,7 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
                                   live_items, num_items, reduce_items, num_reduce_items, seg_q_start, seg_q_len,
                                   seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads,
                                   page_size, max_pages, in_exponent * 1.4426950408889634f, window, q_stride, cap_scale,
-                                  softcap, split_weights, stream};
+                                  softcap, split_weights, sinks, stream};
     switch (head_dim) {
         case 32: return launch_all<32>(a);
         case 64: return launch_all<64>(a);

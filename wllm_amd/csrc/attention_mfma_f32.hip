@@ -39,7 +39,7 @@ paged_attention_f32_kernel(const float* __restrict__ qkv, const float* __restric
                            const int* __restrict__ live_items, float* __restrict__ out,
                            float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                            int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
-                           int q_stride, float cap_scale, float softcap) {
+                           int q_stride, float cap_scale, float softcap, const float* __restrict__ sinks) {
     constexpr int DQ = HD / 4;                  // elements of a lane group's quarter of the head
     constexpr int DT = HD / 16;                 // 16-row tiles of out^T
     constexpr int kQStride = HD + 4;            // floats; rows 4 banks apart: 16 lanes' 16-byte reads meet no conflict
@@ -214,7 +214,9 @@ paged_attention_f32_kernel(const float* __restrict__ qkv, const float* __restric
                 f_of[w] = exp2f((m_of[w] - m_use) * scale_log2e);       // 0 for a wavefront without keys
                 l_all = fmaf(l_of[w], f_of[w], l_all);
             }
-            inv = 1.f / l_all;
+            // a sink: exp(sink of the head) once more in the denominator of a row that is finished here
+            const float sink_term = (sinks && partial_slot < 0) ? exp2f(sinks[head] * 1.4426950408889634f - m_use * scale_log2e) : 0.f;
+            inv = 1.f / (l_all + sink_term);
         }
         if (row_valid) {
 #pragma unroll
@@ -253,7 +255,7 @@ __global__ void __launch_bounds__(HD)
 attention_reduce_f32_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
                             const float* __restrict__ partial_ml, const int* __restrict__ seg_q_start,
                             const int* __restrict__ seg_q_len, float* __restrict__ out, int num_heads,
-                            int num_kv_heads, float scale_log2e) {
+                            int num_kv_heads, float scale_log2e, const float* __restrict__ sinks) {
     constexpr int kQuads = HD / 4;
     const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * kItemInts;
     const int seg = item[0], kvh = item[1], first = item[2], splits = item[3], row0 = item[4];
@@ -297,6 +299,7 @@ attention_reduce_f32_kernel(const int* __restrict__ reduce_items, const float* _
     }
     const int row = row0 + r;
     const int tok = row / group, head = kvh * group + row % group;
+    if (sinks) den += exp2f(sinks[head] * 1.4426950408889634f - m * scale_log2e);
     *reinterpret_cast<float4_t*>(out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD + d) =
         float4_t{num[0] / den, num[1] / den, num[2] / den, num[3] / den};
 }
@@ -319,7 +322,7 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
                                    const int* __restrict__ seg_ctx_len, float* __restrict__ out,
                                    float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                                    int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
-                           int q_stride, float cap_scale, float softcap) {
+                           int q_stride, float cap_scale, float softcap, const float* __restrict__ sinks) {
     constexpr int DQ = HD / 4, DT = HD / 16;
     constexpr int SK = HD + 4, SV = kBlockKeys + 4;
     __shared__ __align__(16) float k_s[kBlockKeys * SK];
@@ -476,6 +479,7 @@ paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* _
         if (g == 0) *reinterpret_cast<float2*>(partial_ml + (slot * 16 + i) * 2) = make_float2(m_run, l);
         return;
     }
+    if (sinks) l += exp2f(sinks[head] * 1.4426950408889634f - m_run * scale_log2e);
     const float inv = 1.f / l;
     float* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
 #pragma unroll
@@ -488,15 +492,15 @@ int launch_f32(const float* qkv, const float* cache, const int* block_tables, co
                int num_items, const int* reduce_items, int num_reduce_items, const int* seg_q_start, const int* seg_q_len,
                float* out, float* partial_o, float* partial_ml, int num_heads, int num_kv_heads, int page_size,
                int max_pages, float scale_log2e, int window, int q_stride, float cap_scale, float softcap,
-               hipStream_t stream) {
+               const float* sinks, hipStream_t stream) {
     if (num_items > 0)
         paged_attention_f32_kernel<HD><<<num_items, 256, 0, stream>>>(qkv, cache, block_tables, items, live_items, out,
                                                                       partial_o, partial_ml, num_heads, num_kv_heads,
                                                                       page_size, max_pages, scale_log2e, window,
-                                                                      q_stride, cap_scale, softcap);
+                                                                      q_stride, cap_scale, softcap, sinks);
     if (num_reduce_items > 0)
         attention_reduce_f32_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile / 4), HD, 0, stream>>>(
-            reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, out, num_heads, num_kv_heads, scale_log2e);
+            reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, out, num_heads, num_kv_heads, scale_log2e, sinks);
     return launch_status();
 }
 
@@ -509,7 +513,7 @@ WLLM_API int wllm_paged_attention_mfma_f32(const float* qkv, const float* cache,
                                            int num_reduce_items, const int* seg_q_start, const int* seg_q_len, float* out,
                                            float* partial_o, float* partial_ml, int num_heads, int num_kv_heads,
                                            int head_dim, int page_size, int max_pages, float scale, int window,
-                                           int q_stride, float softcap, hipStream_t stream) {
+                                           int q_stride, float softcap, const float* sinks, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         num_heads >= (1 << 16))       // an item holds a key/value head and a tile's first row in 16 bits each
         return -1;
@@ -519,7 +523,7 @@ WLLM_API int wllm_paged_attention_mfma_f32(const float* qkv, const float* cache,
 #define LAUNCH(HD)                                                                                                       \
     return launch_f32<HD>(qkv, cache, block_tables, items, live_items, num_items, reduce_items, num_reduce_items,         \
                           seg_q_start, seg_q_len, out, partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
-                          scale_log2e, window, q_stride, cap_scale, softcap, stream)
+                          scale_log2e, window, q_stride, cap_scale, softcap, sinks, stream)
     switch (head_dim) {
         case 32: LAUNCH(32);
         case 64: LAUNCH(64);
@@ -541,7 +545,8 @@ WLLM_API int wllm_paged_attention_prefill_f32(const float* qkv, const float* cac
                                               int num_items, int rows_per_item, const int* seg_q_start, const int* seg_q_len,
                                               const int* seg_ctx_len, float* out, float* partial_o, float* partial_ml,
                                               int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
-                                              float scale, int window, int q_stride, float softcap, hipStream_t stream) {
+                                              float scale, int window, int q_stride, float softcap, const float* sinks,
+                                              hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
         rows_per_item != 64)
         return -1;
@@ -554,7 +559,7 @@ WLLM_API int wllm_paged_attention_prefill_f32(const float* qkv, const float* cac
                                                                           seg_q_len, seg_ctx_len, out, partial_o,        \
                                                                           partial_ml, num_heads, num_kv_heads, page_size, \
                                                                           max_pages, scale_log2e, window, q_stride,      \
-                                                                          cap_scale, softcap);                            \
+                                                                          cap_scale, softcap, sinks);                     \
     break
     switch (head_dim) {
         case 32: LAUNCH(32);

@@ -53,7 +53,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
                                const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                                float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                                int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
-                               int q_stride, float cap_scale, float softcap) {
+                               int q_stride, float cap_scale, float softcap, const float* __restrict__ sinks) {
     constexpr int DC = HD / 32, DT = HD / 16;
     constexpr int SK = PrefillSmem<HD>::kStrideK, SV = PrefillSmem<HD>::kStrideV;
     __shared__ __align__(16) uint16_t k_s[kBlockKeys * SK];
@@ -321,6 +321,8 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             if (g == 0) *reinterpret_cast<float2*>(partial_ml + (slot * 16 + i) * 2) = make_float2(m_run[rt], l);
             continue;
         }
+        // a sink: exp(sink of the head) once more in the denominator of a row that is finished here
+        if (sinks) l += exp2f(sinks[head[rt]] * 1.4426950408889634f - m_run[rt] * scale_log2e);
         const float inv = 1.f / l;
         bf16* orow = out + (static_cast<size_t>(q_start + tok[rt]) * num_heads + head[rt]) * HD;
 #pragma unroll
@@ -389,7 +391,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
                                    const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                                    float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                                    int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window,
-                               int q_stride, float cap_scale, float softcap) {
+                               int q_stride, float cap_scale, float softcap, const float* __restrict__ sinks) {
     constexpr int DC = HD / 32, DT = HD / 16, CPR = HD / 8;       // CPR: 16-byte chunks of a key row
     constexpr int kKeyInstr = kBlockKeys * CPR / 64, kValInstr = HD * 4 / 64;    // wavefront loads per tile
     __shared__ __align__(16) uint16_t k_s0[kBlockKeys * HD], k_s1[kBlockKeys * HD];
@@ -639,6 +641,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
         if (g == 0) *reinterpret_cast<float2*>(partial_ml + (slot * 16 + i) * 2) = make_float2(m_run, l);
         return;
     }
+    if (sinks) l += exp2f(sinks[head] * 1.4426950408889634f - m_run * scale_log2e);
     const float inv = 1.f / l;
     bf16* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
 #pragma unroll
@@ -657,7 +660,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
                                           float* partial_ml, int num_heads,
                                           int num_kv_heads, int head_dim, int page_size, int max_pages, float scale,
                                           int window, int q_stride, float softcap, int split_weights,
-                                          hipStream_t stream) {
+                                          const float* sinks, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
         return -1;
     if (rows_per_item != 64) return -1;
@@ -672,7 +675,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     paged_attention_prefill_dma_kernel<HD, S><<<num_items, kPrefillThreads, 0, stream>>>(                           \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
-        scale_log2e, window, q_stride, cap_scale, softcap)
+        scale_log2e, window, q_stride, cap_scale, softcap, sinks)
         if (head_dim == 64) { LAUNCH_DMA(64); }
         else if (head_dim == 128) { LAUNCH_DMA(128); }
         else { LAUNCH_DMA(256); }
@@ -686,7 +689,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     paged_attention_prefill_kernel<HD, RTW, S><<<num_items, kPrefillThreads, 0, stream>>>(                          \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
-        scale_log2e, window, q_stride, cap_scale, softcap)
+        scale_log2e, window, q_stride, cap_scale, softcap, sinks)
 #define LAUNCH(HD) LAUNCH_RTW(HD, 1)
     switch (head_dim) {
         case 32: LAUNCH(32); break;

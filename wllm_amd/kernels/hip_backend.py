@@ -46,16 +46,16 @@ _SIGNATURES = {
     "wllm_paged_attention_generic_chunk_keys": [],
     "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
-                                  c_int, c_int, c_float, c_int, c_void_p],
+                                  c_int, c_int, c_float, c_int, c_void_p, c_void_p],
     "wllm_paged_attention_mfma_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                      c_float, c_void_p],
+                                      c_float, c_void_p, c_void_p],
     "wllm_paged_attention_prefill_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                         c_int, c_float, c_void_p],
+                                         c_int, c_float, c_void_p, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                                     c_int, c_float, c_int, c_void_p],
+                                     c_int, c_float, c_int, c_void_p, c_void_p],
     "wllm_gemm_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_split_sum": [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -240,8 +240,6 @@ class HipBackend:
         if chunk:
             # the kernels take one integer for the mask: w > 0 a sliding window, -c < 0 chunks of c positions
             window = -int(chunk)
-        if sinks is not None and plan is not None:
-            raise KernelError("paged_attention: the matrix-core kernels have no sinks; give no plan")
         q_stride = qkv.shape[1]         # a row begins with the query heads; this many elements lie between two rows
         if plan is not None:
             if not self.mfma_attention_takes(qkv.dtype, head_dim, page_size):
@@ -252,7 +250,7 @@ class HipBackend:
                         _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.prefill_items), plan.num_prefill,
                         plan.prefill_rows, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
                         _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                        block_tables.shape[1], scale, window, q_stride, softcap, self._stream()),
+                        block_tables.shape[1], scale, window, q_stride, softcap, _ptr(sinks), self._stream()),
                         "paged_attention (prompt portions, matrix cores, float32)")
                 if plan.num_items == 0 and plan.num_reduce == 0:
                     return
@@ -260,7 +258,8 @@ class HipBackend:
                     _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), _ptr(plan.live_items), plan.num_items,
                     _ptr(plan.reduce_items), plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(out),
                     _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                    block_tables.shape[1], scale, window, q_stride, softcap, self._stream()), "paged_attention (matrix cores, float32)")
+                    block_tables.shape[1], scale, window, q_stride, softcap, _ptr(sinks), self._stream()),
+                    "paged_attention (matrix cores, float32)")
                 return
             if plan.num_prefill:
                 self._check(self.lib.wllm_paged_attention_prefill(
@@ -269,7 +268,7 @@ class HipBackend:
                     _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(plan.partial_o),
                     _ptr(plan.partial_ml), num_heads, num_kv_heads,
                     head_dim, page_size, block_tables.shape[1], scale, window, q_stride, softcap, int(exact_weights),
-                    self._stream()), "paged_attention (prompt portions, matrix cores)")
+                    _ptr(sinks), self._stream()), "paged_attention (prompt portions, matrix cores)")
             if plan.num_items == 0 and plan.num_reduce == 0:
                 return
             self._check(self.lib.wllm_paged_attention_mfma(
@@ -277,7 +276,7 @@ class HipBackend:
                 _ptr(plan.live_items), plan.num_items, _ptr(plan.reduce_items),
                 plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
                 _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
-                block_tables.shape[1], scale, window, q_stride, softcap, int(exact_weights), self._stream()),
+                block_tables.shape[1], scale, window, q_stride, softcap, int(exact_weights), _ptr(sinks), self._stream()),
                 "paged_attention (matrix cores)")
             return
         if head_dim % 4 or head_dim > 256:

@@ -312,8 +312,8 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     step.  Token i of it is at position p = ctx_len - q_len + i and sees keys
     max(0, p - window + 1) .. p (window 0: from key 0); with `chunk` c > 0 instead, the keys of its
     own chunk of c positions counted from 0, (p // c) * c .. p.  With `sinks` (float32 [num_heads]) the
-    softmax's denominator holds exp(sinks[h]) once more: a term with no key and no value, not scaled
-    (only the kernels that run without a plan have it).  Query head h uses key/value head
+    softmax's denominator holds exp(sinks[h]) once more: a term with no key and no value, not scaled.
+    Query head h uses key/value head
     h // (num_heads // num_kv_heads).  Scores are scaled by `scale` and then, with `softcap` c > 0,
     bent to c * tanh(score / c); scores, softmax and the weighted sum accumulate in float32.
     The bfloat16 matrix-core kernels round a softmax weight to bfloat16 before they multiply it with the
@@ -347,7 +347,6 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     _need(chunk >= 0 and not (chunk and window), "chunk must not be negative, and excludes a window")
     if sinks is not None:
         _dense(sinks, "sinks", torch.float32, (num_heads,))
-        _need(plan is None, "sinks: only the kernels that run without a plan have them")
     if n:
         backend().paged_attention(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len,
                                   out, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),

@@ -100,8 +100,6 @@ class LatentAttention:
         return 2.0 * tokens * products + 4.0 * s.num_heads * self.rank * keys
 
     def _work_items(self, ctx, page_size: int):
-        if self.sinks is not None:
-            return None             # the kernels that take work items have no sinks
         s = self.spec
         shape = dict(num_heads=s.num_heads, num_kv_heads=1, head_dim=self.rank, page_size=page_size, window=0)
 
