@@ -298,7 +298,7 @@ class EmulatedKernels:
                 carried.copy_(seq[ql:].to(torch.float32))
 
     def ssm_scan(self, xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y, heads, groups,
-                 state_size, head_dim):
+                 state_size, head_dim, steps=None):
         self._count("ssm_scan")
         inner, n_s = heads * head_dim, state_size
         per = heads // groups

@@ -35,7 +35,7 @@ __device__ __forceinline__ void row_stats(const float* row, int hidden, int kind
 }
 
 template <typename TD, typename TO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 norm_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits, size_t split_stride, int d_kind,
                 const float* __restrict__ d_weight, float d_eps, float d_offset, const int* __restrict__ rows,
                 TO* __restrict__ out, int o_kind, const float* __restrict__ o_weight, float o_eps, float o_offset,
@@ -90,8 +90,15 @@ WLLM_API int wllm_norm_add(float* x, const void* delta, int delta_type, int spli
     if (out && o_kind != kNormNone && !o_weight) return -1;
     if (!delta && !out) return 0;
     const size_t smem = sizeof(float) * static_cast<size_t>(hidden);
+    // The few rows of a decode step: a row's time is that of its chain of trips to memory (a stack of partial
+    // sums to add, the stream, the weights), so as many threads as give each two elements; many rows: 256.
+    int threads = 256;
+    if (num_rows <= 256) {
+        threads = (hidden / 2 + 63) / 64 * 64;
+        threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+    }
 #define LAUNCH(TD, TO)                                                                                               \
-    norm_add_kernel<TD, TO><<<num_rows, 256, smem, stream>>>(x, static_cast<const TD*>(delta), splits,                \
+    norm_add_kernel<TD, TO><<<num_rows, threads, smem, stream>>>(x, static_cast<const TD*>(delta), splits,            \
                                                               static_cast<size_t>(split_stride), d_kind, d_weight,   \
                                                               d_eps, d_offset, rows, static_cast<TO*>(out), o_kind,   \
                                                               o_weight, o_eps, o_offset, hidden)
@@ -231,12 +238,72 @@ head_linear_kernel(const T* __restrict__ x, long long x_stride, const T* __restr
     }
 }
 
+// The few rows of a decode step: a workgroup takes one head and 64 outputs, all rows (at most 16).  Thread
+// (o, q) multiplies the q-th quarter of output o's row of w (read once, in runs of consecutive elements) with
+// every row of x, which lies in shared memory; the quarters are added in ascending order, so the sum's order
+// is k ascending within a quarter and quarter by quarter.
+constexpr int kHlFewRows = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_linear_few_kernel(const T* __restrict__ x, long long x_stride, const T* __restrict__ w, T* __restrict__ y,
+                       long long y_stride, int rows, int heads, int outs, int keys) {
+    extern __shared__ float hl_smem[];
+    float* xs = hl_smem;                                  // [rows][keys]
+    float* part = hl_smem + rows * keys;                  // [4][rows][64]
+    const int h = blockIdx.x, o0 = blockIdx.y * kHlOuts;
+    for (int e = threadIdx.x; e < rows * keys; e += blockDim.x) {
+        const int r = e / keys, k = e - r * keys;
+        xs[e] = to_float(x[static_cast<size_t>(r) * x_stride + static_cast<size_t>(h) * keys + k]);
+    }
+    __syncthreads();
+    const int o = threadIdx.x % kHlOuts, q = threadIdx.x / kHlOuts;
+    const int per = (keys + 3) / 4, k_begin = q * per, k_end = min(keys, k_begin + per);
+    float acc[kHlFewRows];
+#pragma unroll
+    for (int r = 0; r < kHlFewRows; ++r) acc[r] = 0.f;
+    if (o0 + o < outs) {
+        const T* wr = w + (static_cast<size_t>(h) * outs + o0 + o) * keys;
+        for (int k = k_begin; k < k_end; ++k) {
+            const float wv = to_float(wr[k]);
+#pragma unroll
+            for (int r = 0; r < kHlFewRows; ++r)
+                if (r < rows) acc[r] = fmaf(xs[r * keys + k], wv, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kHlFewRows; ++r)
+        if (r < rows) part[(q * rows + r) * kHlOuts + o] = acc[r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < rows * kHlOuts; e += blockDim.x) {
+        const int r = e / kHlOuts, oo = e % kHlOuts;
+        if (o0 + oo >= outs) continue;
+        float total = part[r * kHlOuts + oo];
+#pragma unroll
+        for (int qq = 1; qq < 4; ++qq) total += part[(qq * rows + r) * kHlOuts + oo];
+        y[static_cast<size_t>(r) * y_stride + static_cast<size_t>(h) * outs + o0 + oo] = from_float<T>(total);
+    }
+}
+
 WLLM_API int wllm_head_linear(const void* x, long long x_stride, const void* w, void* y, long long y_stride, int is_bf16,
                               int rows, int heads, int outs, int keys, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (heads <= 0 || outs <= 0 || keys <= 0 || heads > 65535) return -1;
     const dim3 grid((rows + kHlRows - 1) / kHlRows, heads, (outs + kHlOuts - 1) / kHlOuts);
     if (grid.z > 65535) return -1;
+    const size_t smem = sizeof(float) * (static_cast<size_t>(rows) * keys + 4 * static_cast<size_t>(rows) * kHlOuts);
+    if (rows <= kHlFewRows && smem <= 48 * 1024) {
+        const dim3 few(heads, (outs + kHlOuts - 1) / kHlOuts);
+        if (is_bf16)
+            head_linear_few_kernel<bf16><<<few, 256, smem, stream>>>(static_cast<const bf16*>(x), x_stride,
+                                                                     static_cast<const bf16*>(w), static_cast<bf16*>(y), y_stride,
+                                                                     rows, heads, outs, keys);
+        else
+            head_linear_few_kernel<float><<<few, 256, smem, stream>>>(static_cast<const float*>(x), x_stride,
+                                                                      static_cast<const float*>(w), static_cast<float*>(y),
+                                                                      y_stride, rows, heads, outs, keys);
+        return launch_status();
+    }
     if (is_bf16)
         head_linear_kernel<bf16><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(w),
                                                            static_cast<bf16*>(y), y_stride, rows, heads, outs, keys);

@@ -86,85 +86,160 @@ WLLM_API int wllm_causal_conv(const void* in, long long in_stride, const float* 
 // ---- the recurrence.  Per head h (group g = h / (heads / groups)), token by token:
 //   dt = softplus(dt_in + dt_bias[h]);  S = exp(-exp(A_log[h]) * dt) * S + dt * B_t x_t^T;  y_t = S^T C_t + D[h] x_t
 // with S [N, P], B_t and C_t [N] of the group, x_t [P] of the head.  xbc [tokens, heads*P + 2*groups*N]
-// holds x, then B, then C.  A workgroup owns (head, segment, 64 columns of P) and walks the segment's
-// tokens in order; lane = column p, the four wavefronts split N, each keeping its rows of S in
-// registers (R a wavefront).  Tokens are staged 16 at a time through shared memory; a token's y is
-// the wavefronts' partial sums added in wavefront order, so it has the same bits whether the token
-// came alone or inside a prompt. ----
+// holds x, then B, then C.  The step sizes and decays of all tokens and heads are made first, by a
+// kernel of their own (`ssm_steps_kernel`: softplus and two exponentials a value, out of the token
+// loop).  Then a workgroup owns (head, segment, 16 columns of P) and walks the segment's tokens in
+// order.  N is cut into 16 slices: a lane is (column, one of four slices), a wavefront four slices,
+// the workgroup's four wavefronts all of them; a lane keeps its R rows of its column of S in
+// registers.  So a head of 64 columns is four workgroups, a prompt's 64 heads fill 256 compute units,
+// and a lane's chain of dependent multiply-adds a token is R long (8 at N = 128).  (8 columns a
+// workgroup and 32 slices: a prompt of 2,048 tokens 654 against 822 us, but 64 decoded tokens 134
+// against 85 us: a lane's 32 bytes of a row of S are half a memory transaction.)  Tokens are staged 16 at a time through shared memory
+// (B, C, x, step, decay), the next 16 fetched into registers meanwhile; a token's y is the slices'
+// partial sums added in a fixed order (within the wavefront, then wavefront by wavefront), so it has
+// the same bits whether the token came alone or inside a prompt. ----
 constexpr int kScanTokens = 16;
 constexpr int kScanWaves = 4;
+constexpr int kScanCols = 16;                       // columns of P a workgroup owns
+constexpr int kScanLaneSlices = kWave / kScanCols;  // slices of N side by side in a wavefront
+constexpr int kScanSlices = kScanWaves * kScanLaneSlices;
+constexpr int kScanFetchers = kWave * kScanWaves / kScanTokens;    // threads that fetch one token's B, C and x of a chunk
+static_assert(kScanFetchers >= kScanCols && (kScanLaneSlices == 4 || kScanLaneSlices == 8),
+              "a token's fetchers cover its columns of x; the lane sums below are for 4 or 8 slices");
 
 __device__ __forceinline__ float softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-template <typename T, int R>
+// steps[0][t][h] = softplus(dt_in[t][h] + dt_bias[h]); steps[1][t][h] = exp(-exp(a_log[h]) * steps[0][t][h])
+template <typename T>
+__global__ void ssm_steps_kernel(const T* __restrict__ dt_in, long long dt_stride, const float* __restrict__ dt_bias,
+                                 const float* __restrict__ a_log, float* __restrict__ steps, int tokens, int heads) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= tokens * heads) return;
+    const int t = e / heads, h = e - t * heads;
+    const float dt = softplus(to_float(dt_in[static_cast<size_t>(t) * dt_stride + h]) + dt_bias[h]);
+    steps[e] = dt;
+    steps[static_cast<size_t>(tokens) * heads + e] = expf(-expf(a_log[h]) * dt);
+}
+
+// VEC: N is a multiple of 4 and so is R, so a lane's rows of B and C are runs of float4 in shared memory.
+// F: elements of B (of C) one of a token's 16 fetchers brings.
+template <typename T, int R, int F, bool VEC>
 __global__ void __launch_bounds__(kWave * kScanWaves)
-ssm_scan_kernel(const T* __restrict__ xbc, const T* __restrict__ dt_in, long long dt_stride,
-                const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
-                float* __restrict__ state, long long state_stride, const int* __restrict__ seg_q_start,
+ssm_scan_kernel(const T* __restrict__ xbc, const float* __restrict__ steps, int tokens,
+                const float* __restrict__ d_skip, float* __restrict__ state, long long state_stride, const int* __restrict__ seg_q_start,
                 const int* __restrict__ seg_q_len, const int* __restrict__ state_slots, float* __restrict__ y, int heads,
                 int groups, int n_state, int p_dim) {
-    extern __shared__ float smem[];
-    const int h = blockIdx.x, seg = blockIdx.y, p0 = blockIdx.z * kWave;
+    extern __shared__ __align__(16) float smem[];
+    const int h = blockIdx.x, seg = blockIdx.y, p0 = blockIdx.z * kScanCols;
     const int q_len = seg_q_len[seg], q_start = seg_q_start[seg];
     if (q_len <= 0) return;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int p = p0 + lane;
+    const int col = lane % kScanCols, slice = wave * kScanLaneSlices + lane / kScanCols;
+    const int p = p0 + col;
     const bool live = p < p_dim;
     const int g = h / (heads / groups);
     const int inner = heads * p_dim, channels = inner + 2 * groups * n_state;
     const int b_col = inner + g * n_state, c_col = inner + groups * n_state + g * n_state;
-    float* b_s = smem;                                   // [kScanTokens][n_state]
-    float* c_s = b_s + kScanTokens * n_state;            // [kScanTokens][n_state]
-    float* x_s = c_s + kScanTokens * n_state;            // [kScanTokens][kWave]
-    float* dt_s = x_s + kScanTokens * kWave;             // [kScanTokens]
+    const int n_pad = (n_state + 3) / 4 * 4;             // a token's row of B (of C) in shared memory
+    float* b_s = smem;                                   // [kScanTokens][n_pad]
+    float* c_s = b_s + kScanTokens * n_pad;              // [kScanTokens][n_pad]
+    float* x_s = c_s + kScanTokens * n_pad;              // [kScanTokens][kScanCols]
+    float* dt_s = x_s + kScanTokens * kScanCols;         // [kScanTokens]
     float* decay_s = dt_s + kScanTokens;                 // [kScanTokens]
-    float* part_s = decay_s + kScanTokens;               // [kScanTokens][kScanWaves][kWave]
+    float* part_s = decay_s + kScanTokens;               // [kScanTokens][kScanWaves][kScanCols]
     float* s_rows = state + static_cast<size_t>(state_slots[seg]) * state_stride + static_cast<size_t>(h) * n_state * p_dim;
-    const int n0 = wave * R;
+    const int n0 = slice * R;
     float s[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) s[i] = (live && n0 + i < n_state) ? s_rows[static_cast<size_t>(n0 + i) * p_dim + p] : 0.f;
-    const float a = -expf(a_log[h]), bias = dt_bias[h], skip = d_skip[h];
+    const float skip = d_skip[h];
+    // What a thread fetches of a chunk of 16 tokens, into registers while the chunk before is worked on:
+    // of token `ft` of the chunk, F elements of B and of C (thread = 16 ft + fq takes the fq-th run), one
+    // element of x, and (the first 16 threads) a token's step size and decay.
+    const int ft = threadIdx.x / kScanFetchers, fq = threadIdx.x % kScanFetchers;
+    float pb[F], pc[F], px = 0.f, pdt = 0.f, pdecay = 0.f;
+    auto fetch = [&](int t0) {
+        const int count = min(kScanTokens, q_len - t0);
+        if (ft < count) {
+            const T* row = xbc + static_cast<size_t>(q_start + t0 + ft) * channels;
+#pragma unroll
+            for (int i = 0; i < F; ++i) {
+                const int n = fq * F + i;
+                pb[i] = n < n_state ? to_float(row[b_col + n]) : 0.f;
+                pc[i] = n < n_state ? to_float(row[c_col + n]) : 0.f;
+            }
+            px = (fq < kScanCols && p0 + fq < p_dim) ? to_float(row[h * p_dim + p0 + fq]) : 0.f;
+        }
+        if (threadIdx.x < count) {
+            const size_t at = static_cast<size_t>(q_start + t0 + threadIdx.x) * heads + h;
+            pdt = steps[at];
+            pdecay = steps[static_cast<size_t>(tokens) * heads + at];
+        }
+    };
+    fetch(0);
     for (int t0 = 0; t0 < q_len; t0 += kScanTokens) {
         const int count = min(kScanTokens, q_len - t0);
         __syncthreads();                                 // the chunk before is read out
-        for (int e = threadIdx.x; e < count * n_state; e += blockDim.x) {
-            const int t = e / n_state, n = e - t * n_state;
-            const T* row = xbc + static_cast<size_t>(q_start + t0 + t) * channels;
-            b_s[e] = to_float(row[b_col + n]);
-            c_s[e] = to_float(row[c_col + n]);
-        }
-        for (int e = threadIdx.x; e < count * kWave; e += blockDim.x) {
-            const int t = e / kWave, l = e % kWave;
-            x_s[e] = p0 + l < p_dim ? to_float(xbc[static_cast<size_t>(q_start + t0 + t) * channels + h * p_dim + p0 + l]) : 0.f;
-        }
-        if (threadIdx.x < count) {
-            const float dt = softplus(to_float(dt_in[static_cast<size_t>(q_start + t0 + threadIdx.x) * dt_stride + h]) + bias);
-            dt_s[threadIdx.x] = dt;
-            decay_s[threadIdx.x] = expf(a * dt);
-        }
-        __syncthreads();
-        for (int t = 0; t < count; ++t) {
-            const float decay = decay_s[t], dx = dt_s[t] * x_s[t * kWave + lane];
-            const float* bt = b_s + t * n_state + n0;
-            const float* ct = c_s + t * n_state + n0;
-            float part = 0.f;
+        if (ft < count) {
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                if (n0 + i < n_state) {
-                    s[i] = fmaf(decay, s[i], dx * bt[i]);
-                    part = fmaf(s[i], ct[i], part);
+            for (int i = 0; i < F; ++i) {
+                const int n = fq * F + i;
+                if (n < n_pad) {
+                    b_s[ft * n_pad + n] = pb[i];
+                    c_s[ft * n_pad + n] = pc[i];
                 }
             }
-            part_s[(t * kScanWaves + wave) * kWave + lane] = part;
+            if (fq < kScanCols) x_s[ft * kScanCols + fq] = px;
+        }
+        if (threadIdx.x < count) {
+            dt_s[threadIdx.x] = pdt;
+            decay_s[threadIdx.x] = pdecay;
         }
         __syncthreads();
-        for (int e = threadIdx.x; e < count * kWave; e += blockDim.x) {
-            const int t = e / kWave, l = e % kWave;
-            if (p0 + l >= p_dim) continue;
-            float total = part_s[(t * kScanWaves) * kWave + l];
+        if (t0 + kScanTokens < q_len) fetch(t0 + kScanTokens);      // in flight while this chunk is worked on
+        // (unrolled: a token's reads of shared memory are asked for while the token before it is multiplied)
+#pragma unroll 4
+        for (int t = 0; t < count; ++t) {
+            const float decay = decay_s[t], dx = dt_s[t] * x_s[t * kScanCols + col];
+            const float* bt = b_s + t * n_pad + n0;
+            const float* ct = c_s + t * n_pad + n0;
+            float part = 0.f;
+            if (VEC) {
 #pragma unroll
-            for (int w = 1; w < kScanWaves; ++w) total += part_s[(t * kScanWaves + w) * kWave + l];
+                for (int i = 0; i < R; i += 4) {
+                    if (n0 + i < n_state) {              // whole groups of four: N and R are multiples of 4
+                        const float4 bv = *reinterpret_cast<const float4*>(bt + i), cv = *reinterpret_cast<const float4*>(ct + i);
+                        s[i] = fmaf(decay, s[i], dx * bv.x);
+                        s[i + 1] = fmaf(decay, s[i + 1], dx * bv.y);
+                        s[i + 2] = fmaf(decay, s[i + 2], dx * bv.z);
+                        s[i + 3] = fmaf(decay, s[i + 3], dx * bv.w);
+                        part = fmaf(s[i], cv.x, part);
+                        part = fmaf(s[i + 1], cv.y, part);
+                        part = fmaf(s[i + 2], cv.z, part);
+                        part = fmaf(s[i + 3], cv.w, part);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    if (n0 + i < n_state) {
+                        s[i] = fmaf(decay, s[i], dx * bt[i]);
+                        part = fmaf(s[i], ct[i], part);
+                    }
+                }
+            }
+            // the wavefront's slices of this column, in a fixed order
+            part = sum_across(sum_across(part, 32), 16);
+            if (kScanLaneSlices == 8) part += row_permuted<0x128>(part);
+            if (lane < kScanCols) part_s[(t * kScanWaves + wave) * kScanCols + col] = part;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < count * kScanCols; e += blockDim.x) {
+            const int t = e / kScanCols, l = e % kScanCols;
+            if (p0 + l >= p_dim) continue;
+            float total = part_s[(t * kScanWaves) * kScanCols + l];
+#pragma unroll
+            for (int w = 1; w < kScanWaves; ++w) total += part_s[(t * kScanWaves + w) * kScanCols + l];
             total = fmaf(skip, x_s[e], total);
             y[static_cast<size_t>(q_start + t0 + t) * inner + h * p_dim + p0 + l] = total;
         }
@@ -176,27 +251,41 @@ ssm_scan_kernel(const T* __restrict__ xbc, const T* __restrict__ dt_in, long lon
     }
 }
 
+// `steps`: scratch of 2 * tokens * heads floats (the step sizes, then the decays).
 WLLM_API int wllm_ssm_scan(const void* xbc, const void* dt_in, long long dt_stride, const float* dt_bias, const float* a_log,
                            const float* d_skip, float* state, long long state_stride, const int* seg_q_start,
-                           const int* seg_q_len, const int* state_slots, float* y, int is_bf16, int segments, int heads,
-                           int groups, int n_state, int p_dim, hipStream_t stream) {
-    if (segments <= 0) return 0;
-    if (heads <= 0 || groups <= 0 || heads % groups != 0 || n_state <= 0 || n_state > 64 * kScanWaves || p_dim <= 0) return -1;
-    if (heads > 65535 * 32 || segments > 65535) return -1;
-    const int r = (n_state + kScanWaves - 1) / kScanWaves;
-    const dim3 grid(heads, segments, (p_dim + kWave - 1) / kWave);
-    const size_t smem = sizeof(float) * (2 * kScanTokens * n_state + kScanTokens * kWave + 2 * kScanTokens +
-                                         kScanTokens * kScanWaves * kWave);
-#define LAUNCH(T, R)                                                                                                \
-    ssm_scan_kernel<T, R><<<grid, kWave * kScanWaves, smem, stream>>>(                                              \
-        static_cast<const T*>(xbc), static_cast<const T*>(dt_in), dt_stride, dt_bias, a_log, d_skip, state,         \
-        state_stride, seg_q_start, seg_q_len, state_slots, y, heads, groups, n_state, p_dim)
-#define LAUNCH_R(T)                        \
-    if (r <= 8) LAUNCH(T, 8);              \
-    else if (r <= 16) LAUNCH(T, 16);       \
-    else if (r <= 32) LAUNCH(T, 32);       \
-    else LAUNCH(T, 64)
-    if (is_bf16) { LAUNCH_R(bf16); } else { LAUNCH_R(float); }
+                           const int* seg_q_len, const int* state_slots, float* y, float* steps, int is_bf16, int tokens,
+                           int segments, int heads, int groups, int n_state, int p_dim, hipStream_t stream) {
+    if (segments <= 0 || tokens <= 0) return 0;
+    if (!steps) return -1;
+    if (heads <= 0 || groups <= 0 || heads % groups != 0 || n_state <= 0 || n_state > 16 * kScanSlices || p_dim <= 0) return -1;
+    if (segments > 65535 || (p_dim + kScanCols - 1) / kScanCols > 65535) return -1;
+    const int r = (n_state + kScanSlices - 1) / kScanSlices;
+    {
+        const int total = tokens * heads, blocks = (total + 255) / 256;
+        if (is_bf16)
+            ssm_steps_kernel<bf16><<<blocks, 256, 0, stream>>>(static_cast<const bf16*>(dt_in), dt_stride, dt_bias, a_log, steps,
+                                                               tokens, heads);
+        else
+            ssm_steps_kernel<float><<<blocks, 256, 0, stream>>>(static_cast<const float*>(dt_in), dt_stride, dt_bias, a_log,
+                                                                steps, tokens, heads);
+        if (const int err = launch_status()) return err;
+    }
+    const int n_pad = (n_state + 3) / 4 * 4;
+    const dim3 grid(heads, segments, (p_dim + kScanCols - 1) / kScanCols);
+    const size_t smem = sizeof(float) * (2 * kScanTokens * n_pad + kScanTokens * kScanCols + 2 * kScanTokens +
+                                         kScanTokens * kScanWaves * kScanCols);
+#define LAUNCH(T, R, V)                                                                                             \
+    ssm_scan_kernel<T, R, (R * kScanSlices + kScanFetchers - 1) / kScanFetchers, V><<<grid, kWave * kScanWaves, smem, stream>>>( \
+        static_cast<const T*>(xbc), steps, tokens, d_skip, state, state_stride, seg_q_start, seg_q_len, state_slots, y, \
+        heads, groups, n_state, p_dim)
+#define LAUNCH_R(T)                                                                          \
+    if (r <= 1) LAUNCH(T, 1, false);                                                         \
+    else if (r <= 2) LAUNCH(T, 2, false);                                                    \
+    else if (r <= 4) { if (n_state % 4 == 0) LAUNCH(T, 4, true); else LAUNCH(T, 4, false); }   \
+    else if (r <= 8) { if (n_state % 4 == 0) LAUNCH(T, 8, true); else LAUNCH(T, 8, false); }   \
+    else { if (n_state % 4 == 0) LAUNCH(T, 16, true); else LAUNCH(T, 16, false); }
+    if (is_bf16) { LAUNCH_R(bf16) } else { LAUNCH_R(float) }
 #undef LAUNCH_R
 #undef LAUNCH
     return launch_status();

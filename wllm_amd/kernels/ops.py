@@ -826,14 +826,17 @@ def causal_conv(inp: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, sta
 
 def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
              state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, state_slots: torch.Tensor,
-             y: torch.Tensor, *, heads: int, groups: int, state_size: int, head_dim: int) -> None:
+             y: torch.Tensor, *, heads: int, groups: int, state_size: int, head_dim: int,
+             steps: Optional[torch.Tensor] = None) -> None:
     """The selective state-space recurrence over each segment's tokens in order, from and into the
     request's carried state.  Per head h (group h // (heads // groups)) and token:
         step = softplus(dt + dt_bias[h]);  S = exp(-exp(a_log[h]) * step) * S + step * B x^T;
         y = S^T C + d_skip[h] * x
     xbc T [n, heads*P + 2*groups*N]: x, then B, then C; dt T [n, heads] (may be a band of a wider row);
     dt_bias, a_log, d_skip float32 [heads]; state float32 [slots, W], whose row state_slots[segment]
-    begins with S as [heads, N, P]; y float32 [n, heads*P].  All of the recurrence is float32."""
+    begins with S as [heads, N, P]; y float32 [n, heads*P].  All of the recurrence is float32.
+    `steps`: float32 [2, n, heads] of scratch for the step sizes and decays (made here if not given; a
+    caller whose step may be captured in a graph gives its own)."""
     _dense(xbc, "xbc", _ACT)
     inner = heads * head_dim
     _need(heads > 0 and groups > 0 and heads % groups == 0, "heads must be a multiple of groups")
@@ -850,9 +853,12 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, a_log: 
     for t, name in ((seg_q_start, "seg_q_start"), (seg_q_len, "seg_q_len"), (state_slots, "state_slots")):
         _dense(t, name, torch.int32, (s,))
     _dense(y, "y", torch.float32, (n, inner))
+    if steps is None:
+        steps = torch.empty((2, n, heads), dtype=torch.float32, device=xbc.device)
+    _dense(steps, "steps", torch.float32, (2, n, heads))
     if n:
         call("ssm_scan", xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y, heads, groups,
-             state_size, head_dim)
+             state_size, head_dim, steps)
 
 
 def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, groups: int,
@@ -978,12 +984,12 @@ def _register_own() -> None:
                     seg_q_start.shape[0], inp.shape[1], weight.shape[1], stream))
     register_op("ssm_scan", entry_point="wllm_ssm_scan",
                 argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
-                          c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
                 launch=lambda fn, stream, xbc, dt, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, state_slots, y,
-                heads, groups, state_size, head_dim: fn(
+                heads, groups, state_size, head_dim, steps: fn(
                     p(xbc), p(dt), dt.stride(0), p(dt_bias), p(a_log), p(d_skip), p(state), state.stride(0), p(seg_q_start),
-                    p(seg_q_len), p(state_slots), p(y), int(xbc.dtype == torch.bfloat16), seg_q_start.shape[0], heads, groups,
-                    state_size, head_dim, stream))
+                    p(seg_q_len), p(state_slots), p(y), p(steps), int(xbc.dtype == torch.bfloat16), xbc.shape[0],
+                    seg_q_start.shape[0], heads, groups, state_size, head_dim, stream))
     register_op("gated_group_norm", entry_point="wllm_gated_group_norm",
                 argtypes=[c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
                 launch=lambda fn, stream, y, z, weight, out, groups, eps: fn(

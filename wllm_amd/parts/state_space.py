@@ -98,7 +98,8 @@ class StateSpaceMixer:
         y = ctx.buffer("ssm_y", (n, self.inner), torch.float32)
         ops.ssm_scan(xbc, row[:, self.inner + self.channels:], self.dt_bias, self.a_log, self.d_skip, state,
                      ctx.seg_q_start, ctx.seg_q_len, ctx.state_slots, y, heads=s.num_heads, groups=s.groups,
-                     state_size=s.state_size, head_dim=s.head_dim)
+                     state_size=s.state_size, head_dim=s.head_dim,
+                     steps=ctx.buffer("ssm_steps", (2, n, s.num_heads), torch.float32))
         out = ctx.buffer("ssm_out", (n, self.inner), h.dtype)
         ops.gated_group_norm(y, row[:, :self.inner], self.norm_w, out, s.norm_groups, s.norm_eps)
         if product_input is not None:
