@@ -8,6 +8,13 @@ import pytest
 from wllm_amd.kernels import attention_plan as ap
 
 
+def lowest(pos, window):
+    """The lowest key a query at `pos` sees: all (0), a window (w > 0) or its own chunk of -w positions (w < 0)."""
+    if window > 0:
+        return max(0, pos - window + 1)
+    return pos - pos % (-window) if window < 0 else 0
+
+
 def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, workgroup_slots=512, tiles_only=False):
     items, reduces, slots, prefill, prefill_rows = ap.build_work_items(
         np.array(q_len), np.array(ctx_len), group, nkv, window, page_size, rows_per_item, workgroup_slots, tiles_only)
@@ -31,7 +38,7 @@ def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, wor
         # the kernel gives each of its four wavefronts one block of 32 keys of an aligned group of 128
         assert kb < ke and kb // 128 == (ke - 1) // 128, (kb, ke)
         first_pos = ctx_len[seg] - q_len[seg]
-        assert kb >= (max(0, first_pos - window + 1) if window > 0 else 0) and ke <= ctx_len[seg]
+        assert kb >= lowest(first_pos, window) and ke <= ctx_len[seg]
         if slot >= 0:
             hold(slot, ("short", n))
         for r in range(row0, min(rows, row0 + 16)):
@@ -43,7 +50,7 @@ def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, wor
         first_pos = ctx_len[seg] - q_len[seg]
         last = min(rows - 1, row0 + prefill_rows - 1)
         b_hi = first_pos + last // group + 1
-        b_lo = max(0, first_pos + row0 // group - window + 1) if window > 0 else 0
+        b_lo = lowest(first_pos + row0 // group, window)
         lo, hi = max(b_lo, kb), min(b_hi, ke)
         assert lo < hi, "an item without keys"
         assert kb % 32 == 0 and ke % 32 == 0
@@ -65,7 +72,7 @@ def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, wor
         for kvh in range(nkv):
             for r in range(q_len[seg] * group):
                 pos = first_pos + r // group
-                lo = max(0, pos - window + 1) if window > 0 else 0
+                lo = lowest(pos, window)
                 pieces = sorted(cover[(seg, kvh, r)])
                 # pieces are disjoint, in order, and hold every key lo..pos
                 assert pieces[0][0] <= lo and pieces[-1][1] > pos, (seg, kvh, r, pieces, lo, pos)
@@ -80,14 +87,14 @@ def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, wor
     return items, reduces, slots, prefill
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(40))
 def test_every_pair_is_covered_once(seed, monkeypatch):
     rng = np.random.default_rng(seed)
     # small targets so that small cases split the way large ones do
     monkeypatch.setattr(ap, "PREFILL_MIN_PIECE", int(rng.choice([1, 4, 12])))
     monkeypatch.setattr(ap, "PREFILL_TABLE_PAGES", int(rng.choice([34, 1024])))
     group, nkv = int(rng.choice([1, 2, 3, 8, 17, 24, 32, 40])), int(rng.choice([1, 2, 3]))
-    window = int(rng.choice([0, 0, 40, 300]))
+    window = int(rng.choice([0, 0, 40, 300, -1, -24, -120, -700]))       # negative: chunks of that many positions
     page_size = int(rng.choice([4, 12, 16, 64]))
     n = int(rng.integers(1, 5))
     q_len = [int(rng.choice([1, 2, 5, 17, 70, 130, 400])) for _ in range(n)]

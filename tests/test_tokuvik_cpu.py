@@ -241,3 +241,25 @@ def test_configurations_drawn_at_random(tmp_path, seed):
         got = replay_and_collect(TraceReplayer(runner), trace)
         runner.cache.check()
     compare_rows(got, reference, relative=5e-4)
+
+
+@pytest.mark.parametrize("layers", [
+    [("mamba", (2, 8, 4, 1, 3, 2), 16), ("mamba", (3, 4, 5, 3, 2, 1), None)],        # no pages at all: state rows alone
+    [("latent", (2, 8, 8, 8, 8), 16)],
+    [("attention", (2, 1, 8, 4), None)],                                             # no mask, no state
+])
+def test_models_of_one_kind_of_mixer(tmp_path, layers):
+    from tokuvik_helpers import attention, config, latent, layer, mamba
+    make = {"mamba": mamba, "latent": latent, "attention": attention}
+    c = dict(page_size=4, seed=5, config=config(40, 16, [layer(make[k](*sizes), ff) for k, sizes, ff in layers]))
+    folder = write_folder(c, str(tmp_path / "m"))
+    requests = requests_for(c, [21, 9, 14])
+    reference = plain_logits(folder, requests, torch.float64)
+    trace = trace_mixed(requests, seed=1, live=2)
+    with ops.use_backend(EmulatedKernels()):
+        model = load_model(folder, "float32", "cpu")
+        runner = ModelRunner.create(model, num_pages=pages_for_max_tokens(max_live_tokens(trace), 4), page_size=4,
+                                    max_requests=2, poison_freed_pages=True)
+        got = replay_and_collect(TraceReplayer(runner), trace)
+        runner.cache.check()
+    compare_rows(got, reference, relative=5e-5)

@@ -101,7 +101,8 @@ def test_band_norms_of_a_wider_row(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n,heads,outs,keys", [(37, 3, 20, 12), (70, 4, 96, 32), (1, 5, 7, 100), (130, 1, 64, 64)])
+@pytest.mark.parametrize("n,heads,outs,keys", [(37, 3, 20, 12), (70, 4, 96, 32), (1, 5, 7, 100), (130, 1, 64, 64), (8, 6, 130, 128),
+                                               (16, 2, 64, 256), (3, 3, 40, 48), (9, 2, 33, 16)])
 def test_products_head_by_head_and_the_gated_lookup(dtype, n, heads, outs, keys):
     g = torch.Generator().manual_seed(n + keys)
     wide = torch.randn(n, heads * keys + 5, generator=g).to(dtype)
@@ -240,6 +241,8 @@ def _attention_problem(dtype, nh, nkv, d, ps, segs, seed, extra_columns):
     (6, 1, 28, 8, 19, True, [(1, 20), (1, 19), (40, 40), (3, 230)]),                        # ... with sinks
     (5, 1, 96, 16, 0, True, [(1, 300), (70, 70), (1, 1), (2, 131)]),                        # sinks, no mask, many heads on one
     (12, 1, 64, 16, 0, True, [(1, 129), (30, 45)]),
+    (10, 1, 20, 8, 0, True, [(1, 150), (21, 40)]),                                          # more heads on a key head than a pass takes
+    (11, 1, 36, 4, 9, True, [(1, 10), (1, 9), (30, 30)]),
     (20, 1, 256, 16, 0, True, [(1, 700), (300, 300), (64, 1000)]),                          # keys cut into pieces: the reduce kernels
     (4, 2, 128, 8, 50, True, [(1, 49), (1, 50), (1, 51), (200, 230)]),
 ])

@@ -244,7 +244,7 @@ head_linear_kernel(const T* __restrict__ x, long long x_stride, const T* __restr
 // is k ascending within a quarter and quarter by quarter.
 constexpr int kHlFewRows = 16;
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 head_linear_few_kernel(const T* __restrict__ x, long long x_stride, const T* __restrict__ w, T* __restrict__ y,
                        long long y_stride, int rows, int heads, int outs, int keys) {
@@ -264,11 +264,40 @@ head_linear_few_kernel(const T* __restrict__ x, long long x_stride, const T* __r
     for (int r = 0; r < kHlFewRows; ++r) acc[r] = 0.f;
     if (o0 + o < outs) {
         const T* wr = w + (static_cast<size_t>(h) * outs + o0 + o) * keys;
-        for (int k = k_begin; k < k_end; ++k) {
-            const float wv = to_float(wr[k]);
+        if (VEC) {
+            // the quarter is a whole number of 16-byte pieces that begin at multiples of 16 bytes: the row of w
+            // streams in as such pieces, several asked for before the first is multiplied
+            constexpr int kPiece = 16 / sizeof(T);
+#pragma unroll 4
+            for (int k = k_begin; k < k_end; k += kPiece) {
+                const uint4 piece = load_streamed(wr + k);
+                float wv[kPiece];
+                if (sizeof(T) == 2) {
+                    const uint32_t words[4] = {piece.x, piece.y, piece.z, piece.w};
 #pragma unroll
-            for (int r = 0; r < kHlFewRows; ++r)
-                if (r < rows) acc[r] = fmaf(xs[r * keys + k], wv, acc[r]);
+                    for (int j = 0; j < 4; ++j) {
+                        wv[2 * j] = __uint_as_float(words[j] << 16);
+                        wv[2 * j + 1] = __uint_as_float(words[j] & 0xffff0000u);
+                    }
+                } else {
+                    wv[0] = __uint_as_float(piece.x);
+                    wv[1] = __uint_as_float(piece.y);
+                    wv[2] = __uint_as_float(piece.z);
+                    wv[3] = __uint_as_float(piece.w);
+                }
+#pragma unroll
+                for (int j = 0; j < kPiece; ++j)
+#pragma unroll
+                    for (int r = 0; r < kHlFewRows; ++r)
+                        if (r < rows) acc[r] = fmaf(xs[r * keys + k + j], wv[j], acc[r]);
+            }
+        } else {
+            for (int k = k_begin; k < k_end; ++k) {
+                const float wv = to_float(wr[k]);
+#pragma unroll
+                for (int r = 0; r < kHlFewRows; ++r)
+                    if (r < rows) acc[r] = fmaf(xs[r * keys + k], wv, acc[r]);
+            }
         }
     }
 #pragma unroll
@@ -294,14 +323,15 @@ WLLM_API int wllm_head_linear(const void* x, long long x_stride, const void* w, 
     const size_t smem = sizeof(float) * (static_cast<size_t>(rows) * keys + 4 * static_cast<size_t>(rows) * kHlOuts);
     if (rows <= kHlFewRows && smem <= 48 * 1024) {
         const dim3 few(heads, (outs + kHlOuts - 1) / kHlOuts);
-        if (is_bf16)
-            head_linear_few_kernel<bf16><<<few, 256, smem, stream>>>(static_cast<const bf16*>(x), x_stride,
-                                                                     static_cast<const bf16*>(w), static_cast<bf16*>(y), y_stride,
-                                                                     rows, heads, outs, keys);
-        else
-            head_linear_few_kernel<float><<<few, 256, smem, stream>>>(static_cast<const float*>(x), x_stride,
-                                                                      static_cast<const float*>(w), static_cast<float*>(y),
-                                                                      y_stride, rows, heads, outs, keys);
+        // whole 16-byte pieces a quarter of a row of w, each at a multiple of 16 bytes
+        const int piece = is_bf16 ? 8 : 4;
+        const bool vec = keys % (4 * piece) == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+#define LAUNCH_FEW(T, V)                                                                                               \
+    head_linear_few_kernel<T, V><<<few, 256, smem, stream>>>(static_cast<const T*>(x), x_stride, static_cast<const T*>(w), \
+                                                             static_cast<T*>(y), y_stride, rows, heads, outs, keys)
+        if (is_bf16) { if (vec) LAUNCH_FEW(bf16, true); else LAUNCH_FEW(bf16, false); }
+        else { if (vec) LAUNCH_FEW(float, true); else LAUNCH_FEW(float, false); }
+#undef LAUNCH_FEW
         return launch_status();
     }
     if (is_bf16)

@@ -54,7 +54,9 @@ class ModelRunner:
             return
         if not self.model.graph_capturable():
             raise ValueError("a part of this model reads the step's arrays on the host; its steps cannot be captured")
-        limit = min(self.model.plan.max_positions, min(g.pool.num_pages - 1 for g in self.cache.groups) * self.cache.page_size)
+        # (a model of recurrent layers alone has no pages: its requests are as long as the model allows)
+        pages = min((g.pool.num_pages - 1 for g in self.cache.groups), default=None)
+        limit = self.model.plan.max_positions if pages is None else min(self.model.plan.max_positions, pages * self.cache.page_size)
         self.graph_max_context = min(max_context or limit, limit)
         if contexts is None:
             contexts = [self.graph_max_context]
