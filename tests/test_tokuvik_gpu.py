@@ -13,7 +13,8 @@ import torch
 
 from helpers import max_live_tokens, replay_and_collect, trace_mixed, trace_portions, trace_tail, trace_whole
 from plain import tokuvik_plain as plain
-from tokuvik_helpers import CONFIGS, compare_rows, plain_logits, random_config, read_folder, requests_for, write_folder
+from tokuvik_helpers import (CONFIGS, compare_rows, middling_config, plain_logits, random_config, read_folder, requests_for,
+                             write_folder)
 from wllm_amd.engine import LLM, ModelRunner
 from wllm_amd.engine.replay import TraceReplayer, pages_for_max_tokens
 from wllm_amd.kernels import ops
@@ -321,6 +322,30 @@ def test_configurations_drawn_at_random(tmp_path, seed):
             model = load_model(folder, dtype, DEV)
             pages = pages_for_max_tokens(max_live_tokens(trace), c["page_size"])
             runner = ModelRunner.create(model, num_pages=pages, page_size=c["page_size"], max_requests=4, poison_freed_pages=True)
+            with torch.inference_mode():
+                got = replay_and_collect(TraceReplayer(runner), trace)
+            runner.cache.check()
+            compare_rows(got, exact, **BOUND[dtype])
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_long_requests_at_middling_sizes(tmp_path, seed):
+    """Widths of some hundred and requests of up to 700 tokens, whole (the library's products, the tiled
+    kernels, blocks of 64 rows in the attention, several tiles of columns in the recurrence) and four at a time."""
+    c = middling_config(300 + seed)
+    folder = write_folder(c, str(tmp_path / "m"))
+    requests = requests_for(c, [700, 129, 300, 65])
+    exact = plain_logits(folder, requests, torch.float64)
+    for dtype in DTYPES:
+        for family in ("whole", "mixed"):
+            trace = FAMILIES[family](requests) if family == "whole" else trace_mixed(requests, seed=seed, portion_sizes=(2, 64, 100, 128, 29))
+            # every tenth row is enough of a long request
+            for step in trace:
+                for e in step["entries"]:
+                    e["want"] = [w for w in e["want"] if w % 10 == 0 or len(e["tokens"]) == 1]
+            model = load_model(folder, dtype, DEV)
+            pages = pages_for_max_tokens(max_live_tokens(trace), 16)
+            runner = ModelRunner.create(model, num_pages=pages, page_size=16, max_requests=4, poison_freed_pages=True)
             with torch.inference_mode():
                 got = replay_and_collect(TraceReplayer(runner), trace)
             runner.cache.check()

@@ -78,6 +78,36 @@ SHARP = dict(page_size=16, seed=13, sharp=True, config=config(200, 96, [
 CONFIGS = {"trio": TRIO, "odd": ODD, "sharp": SHARP}
 
 
+def middling_config(seed: int) -> dict:
+    """Widths of some hundred and heads as a small real model has them: the sizes at which steps of a few hundred
+    rows take the library's products, the tiled kernels and the matrix-core attention."""
+    import random
+    r = random.Random(seed)
+    width = r.choice([256, 384, 512])
+    kv = r.choice([1, 2])
+    dim, vdim = r.choice([(64, 96), (128, 64), (64, 64)])
+    chunk = r.choice([130, 200, 333])
+    heads = kv * r.choice([2, 4])
+    groups = r.choice([1, 2])
+    layers = [
+        layer(attention(heads, kv, dim, vdim, chunk=chunk, scale=dim ** -0.5), r.choice([768, 1024])),
+        layer(latent(r.choice([4, 8]), r.choice([32, 48]), r.choice([32, 64]), r.choice([96, 192]), r.choice([96, 128, 160])), 768),
+        layer(mamba(groups * r.choice([4, 6]), r.choice([32, 64]), r.choice([32, 64, 100]), groups, 4, groups), r.choice([None, 768])),
+        layer(attention(heads * 2, kv, dim, vdim, chunk=r.choice([chunk, None]), scale=dim ** -0.5, kv_from=0), 768),
+    ]
+    r.shuffle(layers)
+    # the reader must come behind the layer it reads: put the owner first again
+    owner = next(i for i, l in enumerate(layers) if l["type"] == "attention" and "kv_from" not in l["mixer"])
+    reader = next(i for i, l in enumerate(layers) if l["mixer"].get("kv_from") is not None)
+    if reader < owner:
+        layers[owner], layers[reader] = layers[reader], layers[owner]
+        owner = reader
+    for l in layers:
+        if l["mixer"].get("kv_from") is not None:
+            l["mixer"]["kv_from"] = owner
+    return dict(page_size=16, seed=seed, config=config(r.choice([1000, 2048]), width, layers, side=r.choice([16, 32]), eps=1e-6))
+
+
 def random_config(seed: int) -> dict:
     """A configuration drawn from what the design allows: any order of mixers, any sizes."""
     import random
