@@ -89,17 +89,20 @@ WLLM_API int wllm_causal_conv(const void* in, long long in_stride, const float* 
 // holds x, then B, then C.  The step sizes and decays of all tokens and heads are made first, by a
 // kernel of their own (`ssm_steps_kernel`: softplus and two exponentials a value, out of the token
 // loop).  Then a workgroup owns (head, segment, 16 columns of P) and walks the segment's tokens in
-// order.  N is cut into 16 slices: a lane is (column, one of four slices), a wavefront four slices,
-// the workgroup's four wavefronts all of them; a lane keeps its R rows of its column of S in
-// registers.  So a head of 64 columns is four workgroups, a prompt's 64 heads fill 256 compute units,
-// and a lane's chain of dependent multiply-adds a token is R long (8 at N = 128).  (8 columns a
-// workgroup and 32 slices: a prompt of 2,048 tokens 654 against 822 us, but 64 decoded tokens 134
-// against 85 us: a lane's 32 bytes of a row of S are half a memory transaction.)  Tokens are staged 16 at a time through shared memory
+// order.  N is cut into 32 slices: a lane is (column, one of four slices), a wavefront four slices,
+// the workgroup's eight wavefronts all of them; a lane keeps its R rows of its column of S in
+// registers.  So a head of 64 columns is four workgroups, a prompt's 64 heads fill 256 compute units
+// with two wavefronts a SIMD (one multiplies while the other waits for shared memory), and a lane's
+// chain of dependent multiply-adds a token is R long (4 at N = 128).  Measured at 64 heads of 64 with
+// 128 rows of state, a prompt of 2,048 tokens / 64 decoded tokens / 8 portions of 256: four wavefronts
+// a workgroup 787 / 83 / 290 us, eight 572 / 88 / 291, sixteen 682 / 113 / 466; eight with 32 tokens a
+// chunk 564 / 105 / 335; 8 columns a workgroup (a lane's 32 bytes of a row of S are half a memory
+// transaction) 654 / 134 / 409.  Tokens are staged 16 at a time through shared memory
 // (B, C, x, step, decay), the next 16 fetched into registers meanwhile; a token's y is the slices'
 // partial sums added in a fixed order (within the wavefront, then wavefront by wavefront), so it has
 // the same bits whether the token came alone or inside a prompt. ----
 constexpr int kScanTokens = 16;
-constexpr int kScanWaves = 4;
+constexpr int kScanWaves = 8;
 constexpr int kScanCols = 16;                       // columns of P a workgroup owns
 constexpr int kScanLaneSlices = kWave / kScanCols;  // slices of N side by side in a wavefront
 constexpr int kScanSlices = kScanWaves * kScanLaneSlices;
